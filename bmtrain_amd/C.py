@@ -1,0 +1,83 @@
+"""Stand-in for BMTrain's compiled extension module ``bmtrain.C`` on the hot path.
+
+The reference registers its launchers with pybind11 (csrc/bind.cpp:3-35); every
+pointer crosses as a Python int and every hyper-parameter as a C float.  This
+module exposes the same callables, with the same names and positional order, on
+top of the C ABI of ``libbmt_hip.so`` (include/bmt_hip.h), loaded with ctypes.
+
+There is no fallback: if the shared library has not been built, importing this
+module raises ImportError; a non-zero status from a launcher raises RuntimeError.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIBRARY_PATH = os.path.join(_HERE, "csrc", "libbmt_hip.so")
+
+if not os.path.exists(LIBRARY_PATH):
+    raise ImportError(
+        f"{LIBRARY_PATH} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}` "
+        "(or `python -c 'import __graft_entry__ as g; g.build()'` from the repository root)"
+    )
+
+_lib = ctypes.CDLL(LIBRARY_PATH)
+
+_i64, _i32, _f, _p = ctypes.c_int64, ctypes.c_int32, ctypes.c_float, ctypes.c_void_p
+_HYPER = [_f] * 8  # beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2
+
+# name -> argument types, in the order of include/bmt_hip.h
+_SIGNATURES = {
+    "has_nan_inf_fp16_launcher": [_i64, _p, _p, _p, _p],
+    "has_nan_inf_bf16_launcher": [_i64, _p, _p, _p, _p],
+    "adam_fp16_launcher": [_i64, _p, _p, _p, _p, _p] + _HYPER + [_p],
+    "adam_bf16_launcher": [_i64, _p, _p, _p, _p, _p] + _HYPER + [_p],
+    "adam_cpu_fp16_launcher": [_i64, _p, _p, _p, _p, _p, _p] + _HYPER,
+    "adam_cpu_bf16_launcher": [_i64, _p, _p, _p, _p, _p, _p] + _HYPER,
+    "to_fp16_from_fp32": [_i64, _p, _p],
+    "to_bf16_from_fp32": [_i64, _p, _p],
+    "cross_entropy_forward_fp16_launcher": [_i32, _i32, _p, _p, _p, _p, _i32, _p],
+    "cross_entropy_forward_bf16_launcher": [_i32, _i32, _p, _p, _p, _p, _i32, _p],
+    "cross_entropy_backward_inplace_fp16_launcher": [_i32, _i32, _p, _p, _p, _i32, _p],
+    "cross_entropy_backward_inplace_bf16_launcher": [_i32, _i32, _p, _p, _p, _i32, _p],
+    "fused_sumexp_fp16_launcher": [_i32, _i32, _p, _p, _p, _p],
+    "fused_sumexp_bf16_launcher": [_i32, _i32, _p, _p, _p, _p],
+    "fused_softmax_inplace_fp16_launcher": [_i32, _i32, _p, _p, _p, _p],
+    "fused_softmax_inplace_bf16_launcher": [_i32, _i32, _p, _p, _p, _p],
+}
+
+_lib.bmt_hip_last_error.restype = ctypes.c_char_p
+_lib.bmt_hip_last_error.argtypes = []
+_lib.is_bf16_supported.restype = ctypes.c_int
+_lib.is_bf16_supported.argtypes = []
+
+
+def last_error() -> str:
+    return (_lib.bmt_hip_last_error() or b"").decode("utf-8", "replace")
+
+
+def _bind(name, argtypes):
+    fn = getattr(_lib, name)
+    fn.argtypes = argtypes
+    fn.restype = ctypes.c_int
+
+    def call(*args):
+        if len(args) != len(argtypes):
+            raise TypeError(f"{name}() takes {len(argtypes)} positional arguments but {len(args)} were given")
+        status = fn(*args)
+        if status != 0:
+            raise RuntimeError(f"{name} failed with status {status}: {last_error()}")
+
+    call.__name__ = name
+    call.__doc__ = f"ctypes binding of `{name}` (include/bmt_hip.h)."
+    return call
+
+
+for _name, _argtypes in _SIGNATURES.items():
+    globals()[_name] = _bind(_name, _argtypes)
+
+
+def is_bf16_supported() -> int:
+    return int(_lib.is_bf16_supported())
+
+
+EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["is_bf16_supported", "bmt_hip_last_error"])

@@ -1,0 +1,319 @@
+// Fused mixed-precision Adam step for gfx950 (MI355X).
+//
+// One streaming pass: per element it reads the fp32 master parameter, the two
+// moments and the 16-bit gradient (14 B for bf16, 12 B for fp16) and writes the
+// fp32 master, the moments and the 16-bit parameter copy (14 B / 12 B).  The
+// kernel is HBM-bound; the design goal is full-width (16 B / lane) coalesced
+// accesses with several independent tiles in flight per wave.
+//
+// Arithmetic (replaces csrc/cuda/adam_cuda.cu:8-72 of the reference).  The
+// expression tree is fixed — this file is compiled with -ffp-contract=off and
+// the only fused multiply-adds are the explicit ones below; `/` and sqrtf are
+// correctly rounded — so that results are reproducible bit-for-bit on a CPU:
+//   bf16:  g  = float(g16) / scale
+//          m' = fma(b1, m, (1-b1)*g)
+//          v' = fma(b2, v, ((1-b2)*g)*g)
+//          p' = fma(-(lr*wd), p, p - ((lr*m')/bc1) / (sqrt(v'/bc2) + eps))
+//   fp16:  g  = float(g16)                      (moments stay multiplied by scale)
+//          m' = fma(b1, float(m16), (1-b1)*g)
+//          v' = fma(b2, v, (((1-b2)*g)*g) / scale)
+//          p' = fma(-(lr*wd), p, p - ((lr*m')/bc1) / (sqrt((v'*scale)/bc2) + eps*scale))
+// This is the reference's expression with the multiply-adds contracted the way
+// its own host compiler contracts the identical CPU loop (adam_cpu.hpp:265-276).
+#include "bmt_device.h"
+#include "bmt_host.h"
+#include "../../include/bmt_hip.h"
+
+#pragma clang fp contract(off)
+
+namespace bmt {
+
+struct AdamHyper {
+    float b1, b2, eps, lr, scale, wd, bc1, bc2;
+};
+
+// Per-element update, bf16 flavour (plain fp32 moments).
+__device__ __forceinline__ void adam_elem_unscaled(float g16f, float &m, float &v, float &p, const AdamHyper &h,
+                                                   float omb1, float omb2, float lrwd) {
+    float g = g16f / h.scale;
+    float mm = __builtin_fmaf(h.b1, m, omb1 * g);
+    float vv = __builtin_fmaf(h.b2, v, (omb2 * g) * g);
+    float den = __builtin_sqrtf(vv / h.bc2) + h.eps;
+    float upd = ((h.lr * mm) / h.bc1) / den;
+    float np = __builtin_fmaf(-lrwd, p, p - upd);
+    m = mm; v = vv; p = np;
+}
+
+// Per-element update, fp16 flavour (moments pre-multiplied by the loss scale).
+__device__ __forceinline__ void adam_elem_scaled(float g, float &m, float &v, float &p, const AdamHyper &h,
+                                                 float omb1, float omb2, float lrwd, float eps_s) {
+    float mm = __builtin_fmaf(h.b1, m, omb1 * g);
+    float vv = __builtin_fmaf(h.b2, v, ((omb2 * g) * g) / h.scale);
+    float den = __builtin_sqrtf((vv * h.scale) / h.bc2) + eps_s;
+    float upd = ((h.lr * mm) / h.bc1) / den;
+    float np = __builtin_fmaf(-lrwd, p, p - upd);
+    m = mm; v = vv; p = np;
+}
+
+// Four elements at once: gradients arrive as two packed dwords.
+template <typename T>
+__device__ __forceinline__ void adam_group_unscaled(u32x2 g, f32x4 &m, f32x4 &v, f32x4 &p, const AdamHyper &h, float omb1,
+                                                    float omb2, float lrwd) {
+    float gm[4] = {lo_f32<T>(g.x), hi_f32<T>(g.x), lo_f32<T>(g.y), hi_f32<T>(g.y)};
+    float ma[4] = {m.x, m.y, m.z, m.w}, va[4] = {v.x, v.y, v.z, v.w}, pa[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+    for (int k = 0; k < 4; k++) adam_elem_unscaled(gm[k], ma[k], va[k], pa[k], h, omb1, omb2, lrwd);
+    m = f32x4{ma[0], ma[1], ma[2], ma[3]};
+    v = f32x4{va[0], va[1], va[2], va[3]};
+    p = f32x4{pa[0], pa[1], pa[2], pa[3]};
+}
+template <typename T>
+__device__ __forceinline__ void adam_group_scaled(u32x2 g, f32x4 &m, f32x4 &v, f32x4 &p, const AdamHyper &h, float omb1,
+                                                  float omb2, float lrwd, float eps_s) {
+    float gm[4] = {lo_f32<T>(g.x), hi_f32<T>(g.x), lo_f32<T>(g.y), hi_f32<T>(g.y)};
+    float ma[4] = {m.x, m.y, m.z, m.w}, va[4] = {v.x, v.y, v.z, v.w}, pa[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+    for (int k = 0; k < 4; k++) adam_elem_scaled(gm[k], ma[k], va[k], pa[k], h, omb1, omb2, lrwd, eps_s);
+    m = f32x4{ma[0], ma[1], ma[2], ma[3]};
+    v = f32x4{va[0], va[1], va[2], va[3]};
+    p = f32x4{pa[0], pa[1], pa[2], pa[3]};
+}
+
+template <typename T>
+__device__ __forceinline__ T ld(const T *p) { return __builtin_nontemporal_load(p); }
+template <typename T>
+__device__ __forceinline__ void st(T *p, T v) { __builtin_nontemporal_store(v, p); }
+
+constexpr int kAdamThreads = 256;
+
+// Vector body, bf16.  `nvec` = number of 4-element groups; every pointer is
+// aligned for its vector type.  A tile is kAdamThreads * UNROLL groups; inside a
+// tile, group u of a thread sits kAdamThreads groups after group u-1, so each
+// load instruction of a wave covers 64 consecutive vectors (1 KiB of fp32).
+template <int UNROLL>
+__global__ __launch_bounds__(kAdamThreads) void adam_bf16_vec_kernel(
+    int64_t nvec, f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, const u32x2 *__restrict__ g16,
+    f32x4 *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h) {
+    const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd;
+    const int64_t tile = (int64_t)kAdamThreads * UNROLL;
+    const int64_t ntiles = (nvec + tile - 1) / tile;
+    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const int64_t base = t * tile + threadIdx.x;
+        f32x4 p[UNROLL], m[UNROLL], v[UNROLL];
+        u32x2 g[UNROLL];
+        if (base - threadIdx.x + tile <= nvec) {
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const int64_t i = base + (int64_t)u * kAdamThreads;
+                g[u] = ld(g16 + i); p[u] = ld(p32 + i); m[u] = ld(mom + i); v[u] = ld(var + i);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const int64_t i = base + (int64_t)u * kAdamThreads;
+                adam_group_unscaled<BFloat16>(g[u], m[u], v[u], p[u], h, omb1, omb2, lrwd);
+                u32x2 o;
+                o.x = pack2<BFloat16>(p[u].x, p[u].y);
+                o.y = pack2<BFloat16>(p[u].z, p[u].w);
+                st(p32 + i, p[u]); st(mom + i, m[u]); st(var + i, v[u]); st(p16 + i, o);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const int64_t i = base + (int64_t)u * kAdamThreads;
+                if (i < nvec) {
+                    u32x2 gg = ld(g16 + i);
+                    f32x4 pp = ld(p32 + i), mm = ld(mom + i), vv = ld(var + i);
+                    adam_group_unscaled<BFloat16>(gg, mm, vv, pp, h, omb1, omb2, lrwd);
+                    u32x2 o;
+                    o.x = pack2<BFloat16>(pp.x, pp.y);
+                    o.y = pack2<BFloat16>(pp.z, pp.w);
+                    st(p32 + i, pp); st(mom + i, mm); st(var + i, vv); st(p16 + i, o);
+                }
+            }
+        }
+    }
+}
+
+// Vector body, fp16: the first moment is a 16-bit array as well.
+template <int UNROLL>
+__global__ __launch_bounds__(kAdamThreads) void adam_fp16_vec_kernel(
+    int64_t nvec, f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, const u32x2 *__restrict__ g16,
+    u32x2 *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h) {
+    const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
+    const int64_t tile = (int64_t)kAdamThreads * UNROLL;
+    const int64_t ntiles = (nvec + tile - 1) / tile;
+    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const int64_t base = t * tile + threadIdx.x;
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const int64_t i = base + (int64_t)u * kAdamThreads;
+            if (i < nvec) {
+                u32x2 gg = ld(g16 + i), mh = ld(mom + i);
+                f32x4 pp = ld(p32 + i), vv = ld(var + i);
+                f32x4 mm;
+                mm.x = lo_f32<Half>(mh.x); mm.y = hi_f32<Half>(mh.x);
+                mm.z = lo_f32<Half>(mh.y); mm.w = hi_f32<Half>(mh.y);
+                adam_group_scaled<Half>(gg, mm, vv, pp, h, omb1, omb2, lrwd, eps_s);
+                u32x2 o, mo;
+                o.x = pack2<Half>(pp.x, pp.y);  o.y = pack2<Half>(pp.z, pp.w);
+                mo.x = pack2<Half>(mm.x, mm.y); mo.y = pack2<Half>(mm.z, mm.w);
+                st(p32 + i, pp); st(var + i, vv); st(mom + i, mo); st(p16 + i, o);
+            }
+        }
+    }
+}
+
+// Element-at-a-time kernels: the unaligned head/tail of a vectorised call, or the
+// whole call when the five arrays do not share one alignment phase.
+__global__ __launch_bounds__(kAdamThreads) void adam_bf16_scalar_kernel(
+    int64_t lo0, int64_t hi0, int64_t lo1, int64_t hi1, float *p32, uint16_t *p16, const uint16_t *g16,
+    float *mom, float *var, AdamHyper h) {
+    const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd;
+    const int64_t n0 = hi0 - lo0, total = n0 + (hi1 - lo1);
+    for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < total; k += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t i = k < n0 ? lo0 + k : lo1 + (k - n0);
+        float p = p32[i], m = mom[i], v = var[i];
+        adam_elem_unscaled(BFloat16::to_f32(g16[i]), m, v, p, h, omb1, omb2, lrwd);
+        p32[i] = p; mom[i] = m; var[i] = v; p16[i] = BFloat16::from_f32(p);
+    }
+}
+__global__ __launch_bounds__(kAdamThreads) void adam_fp16_scalar_kernel(
+    int64_t lo0, int64_t hi0, int64_t lo1, int64_t hi1, float *p32, uint16_t *p16, const uint16_t *g16,
+    uint16_t *mom, float *var, AdamHyper h) {
+    const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
+    const int64_t n0 = hi0 - lo0, total = n0 + (hi1 - lo1);
+    for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < total; k += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t i = k < n0 ? lo0 + k : lo1 + (k - n0);
+        float p = p32[i], m = Half::to_f32(mom[i]), v = var[i];
+        adam_elem_scaled(Half::to_f32(g16[i]), m, v, p, h, omb1, omb2, lrwd, eps_s);
+        p32[i] = p; mom[i] = Half::from_f32(m); var[i] = v; p16[i] = Half::from_f32(p);
+    }
+}
+
+// Splits [0, n) into a scalar head, a vector body of 4-element groups and a scalar
+// tail, given the addresses of the fp32 arrays (16-byte vectors) and the 16-bit
+// arrays (8-byte vectors).  Returns false when the arrays do not share one phase.
+static bool split_for_vectors(int64_t n, const uintptr_t *addr32, int n32, const uintptr_t *addr16, int n16,
+                              int64_t *head, int64_t *nvec) {
+    // Elements to skip until the address is vector-aligned; must agree across arrays.
+    int64_t want = -1;
+    for (int k = 0; k < n32; k++) {
+        if (addr32[k] & 3u) return false;
+        int64_t skip = (int64_t)(((16 - (addr32[k] & 15u)) & 15u) / 4);
+        if (want < 0) want = skip; else if (want != skip) return false;
+    }
+    for (int k = 0; k < n16; k++) {
+        if (addr16[k] & 1u) return false;
+        int64_t skip = (int64_t)(((8 - (addr16[k] & 7u)) & 7u) / 2);
+        if (want < 0) want = skip; else if (want != skip) return false;
+    }
+    if (want > n) want = n;
+    *head = want;
+    *nvec = (n - want) / 4;
+    return true;
+}
+
+static int adam_grid(int64_t ntiles) {
+    // Enough resident workgroups to cover memory latency on every CU, few enough that
+    // each one streams many tiles; the default can be overridden for experiments.
+    static const int per_cu = env_int("BMT_ADAM_BLOCKS_PER_CU", 8);
+    int64_t cap = (int64_t)device_cu_count() * per_cu;
+    return (int)(ntiles < cap ? (ntiles < 1 ? 1 : ntiles) : cap);
+}
+
+template <int UNROLL>
+static hipError_t launch_bf16(int64_t n, float *p32, uint16_t *p16, const uint16_t *g, float *m, float *v,
+                              const AdamHyper &h, hipStream_t s) {
+    uintptr_t a32[3] = {(uintptr_t)p32, (uintptr_t)m, (uintptr_t)v};
+    uintptr_t a16[2] = {(uintptr_t)p16, (uintptr_t)g};
+    int64_t head = 0, nvec = 0;
+    if (!split_for_vectors(n, a32, 3, a16, 2, &head, &nvec)) {
+        int64_t blocks = (n + kAdamThreads - 1) / kAdamThreads;
+        int64_t cap = (int64_t)device_cu_count() * 32;
+        hipLaunchKernelGGL(adam_bf16_scalar_kernel, dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(kAdamThreads), 0, s,
+                           (int64_t)0, n, (int64_t)0, (int64_t)0, p32, p16, g, m, v, h);
+        return hipGetLastError();
+    }
+    if (nvec > 0) {
+        const int64_t tile = (int64_t)kAdamThreads * UNROLL;
+        const int64_t ntiles = (nvec + tile - 1) / tile;
+        hipLaunchKernelGGL(adam_bf16_vec_kernel<UNROLL>, dim3(adam_grid(ntiles)), dim3(kAdamThreads), 0, s, nvec,
+                           (f32x4 *)(p32 + head), (u32x2 *)(p16 + head), (const u32x2 *)(g + head),
+                           (f32x4 *)(m + head), (f32x4 *)(v + head), h);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    const int64_t tail_lo = head + nvec * 4;
+    if (head > 0 || tail_lo < n) {
+        hipLaunchKernelGGL(adam_bf16_scalar_kernel, dim3(1), dim3(kAdamThreads), 0, s, (int64_t)0, head, tail_lo, n,
+                           p32, p16, g, m, v, h);
+        return hipGetLastError();
+    }
+    return hipSuccess;
+}
+
+template <int UNROLL>
+static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16_t *g, uint16_t *m, float *v,
+                              const AdamHyper &h, hipStream_t s) {
+    uintptr_t a32[2] = {(uintptr_t)p32, (uintptr_t)v};
+    uintptr_t a16[3] = {(uintptr_t)p16, (uintptr_t)g, (uintptr_t)m};
+    int64_t head = 0, nvec = 0;
+    if (!split_for_vectors(n, a32, 2, a16, 3, &head, &nvec)) {
+        int64_t blocks = (n + kAdamThreads - 1) / kAdamThreads;
+        int64_t cap = (int64_t)device_cu_count() * 32;
+        hipLaunchKernelGGL(adam_fp16_scalar_kernel, dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(kAdamThreads), 0, s,
+                           (int64_t)0, n, (int64_t)0, (int64_t)0, p32, p16, g, m, v, h);
+        return hipGetLastError();
+    }
+    if (nvec > 0) {
+        const int64_t tile = (int64_t)kAdamThreads * UNROLL;
+        const int64_t ntiles = (nvec + tile - 1) / tile;
+        hipLaunchKernelGGL(adam_fp16_vec_kernel<UNROLL>, dim3(adam_grid(ntiles)), dim3(kAdamThreads), 0, s, nvec,
+                           (f32x4 *)(p32 + head), (u32x2 *)(p16 + head), (const u32x2 *)(g + head),
+                           (u32x2 *)(m + head), (f32x4 *)(v + head), h);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    const int64_t tail_lo = head + nvec * 4;
+    if (head > 0 || tail_lo < n) {
+        hipLaunchKernelGGL(adam_fp16_scalar_kernel, dim3(1), dim3(kAdamThreads), 0, s, (int64_t)0, head, tail_lo, n,
+                           p32, p16, g, m, v, h);
+        return hipGetLastError();
+    }
+    return hipSuccess;
+}
+
+}  // namespace bmt
+
+using namespace bmt;
+
+extern "C" int adam_bf16_launcher(int64_t n, void *param_fp32, void *param_bf16, const void *g_bf16, void *m_fp32,
+                                  void *v_fp32, float beta1, float beta2, float eps, float lr, float scale,
+                                  float weight_decay, float bias_correction1, float bias_correction2, void *stream) {
+    if (n <= 0) return 0;  // adam_cuda.cu:118
+    if (!param_fp32 || !param_bf16 || !g_bf16 || !m_fp32 || !v_fp32) return fail(-1, "adam_bf16_launcher: null pointer");
+    AdamHyper h{beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2};
+    static const int unroll = env_int("BMT_ADAM_UNROLL", 2);
+    hipError_t e;
+    if (unroll == 1)
+        e = launch_bf16<1>(n, (float *)param_fp32, (uint16_t *)param_bf16, (const uint16_t *)g_bf16, (float *)m_fp32,
+                           (float *)v_fp32, h, (hipStream_t)stream);
+    else if (unroll == 4)
+        e = launch_bf16<4>(n, (float *)param_fp32, (uint16_t *)param_bf16, (const uint16_t *)g_bf16, (float *)m_fp32,
+                           (float *)v_fp32, h, (hipStream_t)stream);
+    else
+        e = launch_bf16<2>(n, (float *)param_fp32, (uint16_t *)param_bf16, (const uint16_t *)g_bf16, (float *)m_fp32,
+                           (float *)v_fp32, h, (hipStream_t)stream);
+    return e == hipSuccess ? 0 : fail((int)e, "adam_bf16_launcher", e);
+}
+
+extern "C" int adam_fp16_launcher(int64_t n, void *param_fp32, void *param_fp16, const void *g_fp16, void *m_fp16,
+                                  void *v_fp32, float beta1, float beta2, float eps, float lr, float scale,
+                                  float weight_decay, float bias_correction1, float bias_correction2, void *stream) {
+    if (n <= 0) return 0;  // adam_cuda.cu:91
+    if (!param_fp32 || !param_fp16 || !g_fp16 || !m_fp16 || !v_fp32) return fail(-1, "adam_fp16_launcher: null pointer");
+    AdamHyper h{beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2};
+    hipError_t e = launch_fp16<2>(n, (float *)param_fp32, (uint16_t *)param_fp16, (const uint16_t *)g_fp16,
+                                  (uint16_t *)m_fp16, (float *)v_fp32, h, (hipStream_t)stream);
+    return e == hipSuccess ? 0 : fail((int)e, "adam_fp16_launcher", e);
+}

@@ -1,0 +1,84 @@
+// Device-side helpers shared by the gfx950 kernels: 16-bit float conversions,
+// vector types, wave64 / workgroup reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bmt {
+
+typedef float    f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;  // gfx950 wavefront
+
+// ---- element types -------------------------------------------------------
+// A 16-bit float travels as its bit pattern; the tag type picks the converters.
+struct Half {  // IEEE binary16
+    static __device__ __forceinline__ float to_f32(uint16_t b) {
+        return (float)__builtin_bit_cast(_Float16, b);          // exact, subnormals kept
+    }
+    static __device__ __forceinline__ uint16_t from_f32(float f) {
+        return __builtin_bit_cast(uint16_t, (_Float16)f);        // v_cvt_f16_f32, round-nearest-even
+    }
+    static constexpr uint32_t kExpMask2 = 0x7C007C00u;   // exponent field of both halves of a dword
+    static constexpr uint32_t kExpCarry2 = 0x04000400u;  // exponent all-ones + this carries into bit 15
+};
+struct BFloat16 {  // bfloat16 = upper half of binary32
+    static __device__ __forceinline__ float to_f32(uint16_t b) {
+        return __builtin_bit_cast(float, (uint32_t)b << 16);
+    }
+    static __device__ __forceinline__ uint16_t from_f32(float f) {  // round-nearest-even, NaN quieted
+        uint32_t u = __builtin_bit_cast(uint32_t, f);
+        uint32_t r = u + 0x7FFFu + ((u >> 16) & 1u);
+        uint32_t q = u | 0x00400000u;
+        return (uint16_t)(((u & 0x7FFFFFFFu) > 0x7F800000u ? q : r) >> 16);
+    }
+    static constexpr uint32_t kExpMask2 = 0x7F807F80u;
+    static constexpr uint32_t kExpCarry2 = 0x00800080u;
+};
+
+template <typename T>
+__device__ __forceinline__ float lo_f32(uint32_t packed) { return T::to_f32((uint16_t)(packed & 0xFFFFu)); }
+template <typename T>
+__device__ __forceinline__ float hi_f32(uint32_t packed) { return T::to_f32((uint16_t)(packed >> 16)); }
+template <>
+__device__ __forceinline__ float lo_f32<BFloat16>(uint32_t packed) { return __builtin_bit_cast(float, packed << 16); }
+template <>
+__device__ __forceinline__ float hi_f32<BFloat16>(uint32_t packed) { return __builtin_bit_cast(float, packed & 0xFFFF0000u); }
+
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    return (uint32_t)T::from_f32(lo) | ((uint32_t)T::from_f32(hi) << 16);
+}
+
+// ---- wave64 reductions ----------------------------------------------------
+// Butterfly over the 64 lanes: every lane ends with the full result.
+__device__ __forceinline__ float wave_allreduce_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+__device__ __forceinline__ float wave_allreduce_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// Workgroup all-reduce through LDS: one float per wave, every thread returns the result.
+// `slots` must hold blockDim.x / 64 floats and may be reused after the call returns
+// only after another barrier.
+template <bool IsMax>
+__device__ __forceinline__ float block_allreduce(float v, float *slots) {
+    v = IsMax ? wave_allreduce_max(v) : wave_allreduce_sum(v);
+    const int nwaves = (int)(blockDim.x / kWave);
+    if (nwaves == 1) return v;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (lane == 0) slots[wave] = v;
+    __syncthreads();
+    float r = slots[0];
+    for (int w = 1; w < nwaves; w++) r = IsMax ? fmaxf(r, slots[w]) : r + slots[w];
+    return r;
+}
+
+}  // namespace bmt

@@ -1,0 +1,434 @@
+// Fused cross-entropy forward / in-place backward for gfx950 (MI355X), plus the two
+// row helpers used by the vocabulary-parallel loss.  Replaces
+// csrc/cuda/cross_entropy.cu of the reference.
+//
+// Forward (reference kernels :9-43, :63-101) per row r of the [m, n] logits:
+//   M = max(max_i x_i, -1e6);  S = sum_i expf(x_i - M) + 1e-10
+//   softmax[r, i] = to16(expf(x_i - M) / S)
+//   out[r] = target[r] != ignore ? (-x[target[r]] + M) + logf(S) : 0
+// The reference walks each row three times from global memory.  Here a row is read
+// from HBM once, as 16-byte vectors, into the registers of the workgroup that owns
+// it; the maximum, the exponentials (kept in fp32 registers when they fit, else
+// recomputed from the packed row), the sum and the quotient all work on registers,
+// and the softmax goes out as 16-byte vectors.  Reductions are a wave64 butterfly
+// followed by one LDS slot per wave.  Rows whose length is not a multiple of 8 or
+// whose base is not 16-byte aligned, and rows too long for the register file, take a
+// three-sweep kernel with element loads that relies on L2 for the re-reads.
+//
+// Backward (reference kernels :46-60, :104-121), element-wise and in place on the
+// stored softmax: x[r, i] = to16((x[r, i] - (i == target[r])) * grad_output[r]).
+#include "bmt_device.h"
+#include "bmt_host.h"
+#include "../../include/bmt_hip.h"
+
+namespace bmt {
+
+template <typename T> __device__ __forceinline__ uint32_t neg_inf2();
+template <> __device__ __forceinline__ uint32_t neg_inf2<Half>() { return 0xFC00FC00u; }
+template <> __device__ __forceinline__ uint32_t neg_inf2<BFloat16>() { return 0xFF80FF80u; }
+
+__device__ __forceinline__ float add_tiny(float s) { return (float)((double)s + 1e-10); }  // cross_entropy.cu:28
+
+// Loss of one row; an out-of-range target that is not ignore_index yields NaN instead
+// of the reference's out-of-bounds read.
+template <typename T>
+__device__ __forceinline__ float row_loss(const uint16_t *row, int32_t n, int32_t t, int32_t ignore_index, float M,
+                                          float S) {
+    if (t == ignore_index) return 0.f;
+    if (t < 0 || t >= n) return __builtin_nanf("");
+    return (-T::to_f32(row[t]) + M) + logf(S);
+}
+
+// ---- forward, register-resident row ------------------------------------------
+// One workgroup of THREADS lanes per row; lane t owns vectors t, t+THREADS, ...
+// (CHUNKS of them, 8 elements each).  KEEP_EXP: hold the 8*CHUNKS exponentials in
+// fp32 registers between the sum and the quotient; otherwise recompute them.
+template <typename T, int THREADS, int CHUNKS, bool KEEP_EXP>
+__global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
+    int32_t n, int32_t nvec, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
+    uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
+    __shared__ float slots[2][THREADS / kWave];
+    const int64_t row = blockIdx.x;
+    const u32x4 *xr = (const u32x4 *)(x + row * n);
+    u32x4 *sr = (u32x4 *)(softmax + row * n);
+    const int tid = threadIdx.x;
+
+    u32x4 w[CHUNKS];
+    const uint32_t pad = neg_inf2<T>();
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+        const int j = c * THREADS + tid;
+        if (j < nvec) w[c] = __builtin_nontemporal_load(xr + j);
+        else { w[c].x = pad; w[c].y = pad; w[c].z = pad; w[c].w = pad; }
+    }
+
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            mx = fmaxf(lo_f32<T>(w[c][k]), mx);
+            mx = fmaxf(hi_f32<T>(w[c][k]), mx);
+        }
+        if (!KEEP_EXP) __builtin_amdgcn_sched_barrier(0);
+    }
+    const float M = fmaxf(block_allreduce<true>(mx, slots[0]), -1e6f);
+
+    float e[KEEP_EXP ? CHUNKS : 1][8];
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const float a = expf(lo_f32<T>(w[c][k]) - M), b = expf(hi_f32<T>(w[c][k]) - M);
+            sum += a; sum += b;
+            if (KEEP_EXP) { e[c][2 * k] = a; e[c][2 * k + 1] = b; }
+        }
+        // Long rows live in most of the register file: keep the scheduler from overlapping
+        // the temporaries of many chunks, which would spill the row.
+        if (!KEEP_EXP) __builtin_amdgcn_sched_barrier(0);
+    }
+    const float S = add_tiny(block_allreduce<false>(sum, slots[1]));
+
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+        const int j = c * THREADS + tid;
+        if (j < nvec) {
+            u32x4 o;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const float a = KEEP_EXP ? e[c][2 * k] : expf(lo_f32<T>(w[c][k]) - M);
+                const float b = KEEP_EXP ? e[c][2 * k + 1] : expf(hi_f32<T>(w[c][k]) - M);
+                o[k] = pack2<T>(a / S, b / S);
+            }
+            __builtin_nontemporal_store(o, sr + j);
+        }
+        if (!KEEP_EXP) __builtin_amdgcn_sched_barrier(0);
+    }
+    if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, S);
+}
+
+// ---- forward, long rows: registers + LDS ---------------------------------------
+// A row of up to (REG + LDSC) * 8192 elements is held on chip by one 1024-lane
+// workgroup: REG vectors per lane stay in registers, LDSC more per lane sit in LDS
+// (lane-contiguous 16-byte slots, conflict-free).  Used when the row does not fit
+// the register file alone; exponentials are recomputed in the output sweep.
+template <typename T>
+__device__ __forceinline__ void vec_max(const u32x4 &w, float &mx) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) { mx = fmaxf(lo_f32<T>(w[k]), mx); mx = fmaxf(hi_f32<T>(w[k]), mx); }
+}
+template <typename T>
+__device__ __forceinline__ void vec_sumexp(const u32x4 &w, float M, float &sum) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) { sum += expf(lo_f32<T>(w[k]) - M); sum += expf(hi_f32<T>(w[k]) - M); }
+}
+template <typename T>
+__device__ __forceinline__ u32x4 vec_softmax(const u32x4 &w, float M, float S) {
+    u32x4 o;
+#pragma unroll
+    for (int k = 0; k < 4; k++) o[k] = pack2<T>(expf(lo_f32<T>(w[k]) - M) / S, expf(hi_f32<T>(w[k]) - M) / S);
+    return o;
+}
+
+constexpr int kLongThreads = 1024;
+template <typename T, int REG, int LDSC>
+__global__ __launch_bounds__(kLongThreads) void ce_forward_long_kernel(
+    int32_t n, int32_t nvec, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
+    uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
+    extern __shared__ u32x4 staged[];  // LDSC * 1024 vectors
+    __shared__ float slots[2][kLongThreads / kWave];
+    const int64_t row = blockIdx.x;
+    const u32x4 *xr = (const u32x4 *)(x + row * n);
+    u32x4 *sr = (u32x4 *)(softmax + row * n);
+    const int tid = threadIdx.x;
+    const uint32_t pad = neg_inf2<T>();
+    const u32x4 pad4 = {pad, pad, pad, pad};
+
+    u32x4 w[REG];
+#pragma unroll
+    for (int c = 0; c < REG; c++) {
+        const int j = c * kLongThreads + tid;
+        w[c] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
+    }
+#pragma unroll
+    for (int c = 0; c < LDSC; c++) {
+        const int j = (REG + c) * kLongThreads + tid;
+        staged[c * kLongThreads + tid] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
+    }
+    // Every lane reads back only the LDS slots it wrote itself: no barrier is needed for them.
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < REG; c++) vec_max<T>(w[c], mx);
+#pragma unroll 2
+    for (int c = 0; c < LDSC; c++) vec_max<T>(staged[c * kLongThreads + tid], mx);
+    const float M = fmaxf(block_allreduce<true>(mx, slots[0]), -1e6f);
+
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < REG; c++) { vec_sumexp<T>(w[c], M, sum); __builtin_amdgcn_sched_barrier(0); }
+#pragma unroll 1
+    for (int c = 0; c < LDSC; c++) vec_sumexp<T>(staged[c * kLongThreads + tid], M, sum);
+    const float S = add_tiny(block_allreduce<false>(sum, slots[1]));
+
+#pragma unroll
+    for (int c = 0; c < REG; c++) {
+        const int j = c * kLongThreads + tid;
+        if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(w[c], M, S), sr + j);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll 1
+    for (int c = 0; c < LDSC; c++) {
+        const int j = (REG + c) * kLongThreads + tid;
+        if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(staged[c * kLongThreads + tid], M, S), sr + j);
+    }
+    if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, S);
+}
+
+// ---- forward, any row length / alignment ---------------------------------------
+// One workgroup per row, three sweeps with 2-byte loads (max; sum of exponentials;
+// quotient).  The second and third sweep re-read the row through the caches.
+constexpr int kSweepThreads = 256;
+template <typename T>
+__global__ __launch_bounds__(kSweepThreads) void ce_forward_sweep_kernel(
+    int32_t n, const uint16_t *__restrict__ x, const int32_t *__restrict__ target, uint16_t *__restrict__ softmax,
+    float *__restrict__ out, int32_t ignore_index) {
+    __shared__ float slots[2][kSweepThreads / kWave];
+    const int64_t row = blockIdx.x;
+    const uint16_t *xr = x + row * n;
+    uint16_t *sr = softmax + row * n;
+    float mx = -INFINITY;
+    for (int i = threadIdx.x; i < n; i += kSweepThreads) mx = fmaxf(T::to_f32(xr[i]), mx);
+    const float M = fmaxf(block_allreduce<true>(mx, slots[0]), -1e6f);
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < n; i += kSweepThreads) sum += expf(T::to_f32(xr[i]) - M);
+    const float S = add_tiny(block_allreduce<false>(sum, slots[1]));
+    for (int i = threadIdx.x; i < n; i += kSweepThreads) sr[i] = T::from_f32(expf(T::to_f32(xr[i]) - M) / S);
+    if (threadIdx.x == 0) out[row] = row_loss<T>(xr, n, target[row], ignore_index, M, S);
+}
+
+// ---- element-wise kernels over the flat [m * n] array -----------------------------
+// OP 0: backward in place.  OP 1: softmax in place from given max / sum.
+constexpr int kFlatThreads = 256;
+constexpr int kFlatUnroll = 4;
+
+template <typename T, int OP>
+__device__ __forceinline__ float flat_elem(float s, bool is_target, float a, float b) {
+    if (OP == 0) return is_target ? (s - 1.f) * a : s * a;  // a = grad_output[r]
+    return expf(s - a) / b;                                 // a = max, b = sum
+}
+
+template <typename T, int OP>
+__global__ __launch_bounds__(kFlatThreads) void ce_flat_vec_kernel(
+    int32_t nvec, int64_t total_vec, uint16_t *__restrict__ x, const float *__restrict__ row_a,
+    const float *__restrict__ row_b, const int32_t *__restrict__ target) {
+    u32x4 *xv = (u32x4 *)x;
+    const int64_t tile = (int64_t)kFlatThreads * kFlatUnroll;
+    const int64_t ntiles = (total_vec + tile - 1) / tile;
+    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const int64_t start = t * tile;
+        const int64_t row0 = start / nvec;
+        const uint32_t col0 = (uint32_t)(start - row0 * nvec);
+        u32x4 w[kFlatUnroll];
+        bool ok[kFlatUnroll];
+#pragma unroll
+        for (int u = 0; u < kFlatUnroll; u++) {
+            const int64_t g = start + (int64_t)u * kFlatThreads + threadIdx.x;
+            ok[u] = g < total_vec;
+            if (ok[u]) w[u] = __builtin_nontemporal_load(xv + g);
+        }
+#pragma unroll
+        for (int u = 0; u < kFlatUnroll; u++) {
+            if (!ok[u]) continue;
+            const int64_t g = start + (int64_t)u * kFlatThreads + threadIdx.x;
+            const uint32_t off = col0 + (uint32_t)(u * kFlatThreads + threadIdx.x);
+            const uint32_t dr = off / (uint32_t)nvec;
+            const int64_t row = row0 + dr;
+            const int32_t col = (int32_t)(off - dr * (uint32_t)nvec) * 8;
+            const float a = row_a[row];
+            const float b = OP == 1 ? row_b[row] : 0.f;
+            const int32_t tk = OP == 0 ? target[row] - col : -1;  // position of the target inside this vector
+            u32x4 o;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const float lo = flat_elem<T, OP>(lo_f32<T>(w[u][k]), tk == 2 * k, a, b);
+                const float hi = flat_elem<T, OP>(hi_f32<T>(w[u][k]), tk == 2 * k + 1, a, b);
+                o[k] = pack2<T>(lo, hi);
+            }
+            __builtin_nontemporal_store(o, xv + g);
+        }
+    }
+}
+
+template <typename T, int OP>
+__global__ __launch_bounds__(kFlatThreads) void ce_flat_scalar_kernel(
+    int32_t n, int64_t total, uint16_t *__restrict__ x, const float *__restrict__ row_a,
+    const float *__restrict__ row_b, const int32_t *__restrict__ target) {
+    for (int64_t g = (int64_t)blockIdx.x * kFlatThreads + threadIdx.x; g < total; g += (int64_t)gridDim.x * kFlatThreads) {
+        const int64_t row = g / n;
+        const int32_t col = (int32_t)(g - row * n);
+        const float a = row_a[row];
+        const float b = OP == 1 ? row_b[row] : 0.f;
+        const bool is_t = OP == 0 ? (target[row] == col) : false;
+        x[g] = T::from_f32(flat_elem<T, OP>(T::to_f32(x[g]), is_t, a, b));
+    }
+}
+
+// ---- row sum of exponentials given the row maximum ---------------------------------
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kSweepThreads) void sumexp_kernel(int32_t n, const uint16_t *__restrict__ x,
+                                                               const float *__restrict__ row_max,
+                                                               float *__restrict__ row_sum) {
+    __shared__ float slots[kSweepThreads / kWave];
+    const int64_t row = blockIdx.x;
+    const float M = row_max[row];
+    float sum = 0.f;
+    if (VEC) {
+        const u32x4 *xr = (const u32x4 *)(x + row * n);
+        const int nvec = n / 8;
+        for (int j = threadIdx.x; j < nvec; j += kSweepThreads) {
+            const u32x4 w = __builtin_nontemporal_load(xr + j);
+#pragma unroll
+            for (int k = 0; k < 4; k++) { sum += expf(lo_f32<T>(w[k]) - M); sum += expf(hi_f32<T>(w[k]) - M); }
+        }
+    } else {
+        const uint16_t *xr = x + row * n;
+        for (int i = threadIdx.x; i < n; i += kSweepThreads) sum += expf(T::to_f32(xr[i]) - M);
+    }
+    sum = block_allreduce<false>(sum, slots);
+    if (threadIdx.x == 0) row_sum[row] = sum;
+}
+
+// ---- host side ------------------------------------------------------------------
+static bool rows_vectorisable(int32_t n, const void *a, const void *b = nullptr) {
+    return (n % 8 == 0) && (((uintptr_t)a & 15u) == 0) && (b == nullptr || ((uintptr_t)b & 15u) == 0);
+}
+
+static int flat_grid(int64_t work_items, int threads_times_unroll) {
+    const int64_t tiles = (work_items + threads_times_unroll - 1) / threads_times_unroll;
+    const int64_t cap = (int64_t)device_cu_count() * 16;
+    return (int)(tiles < 1 ? 1 : (tiles < cap ? tiles : cap));
+}
+
+#define BMT_CE_ROW(THREADS, CHUNKS, KEEP)                                                                          \
+    hipLaunchKernelGGL((ce_forward_row_kernel<T, THREADS, CHUNKS, KEEP>), dim3((unsigned)m), dim3(THREADS), 0, s, n, nvec, \
+                       (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,     \
+                       ignore_index)
+
+// Dynamic LDS beyond 64 KiB has to be allowed per kernel once.
+#define BMT_CE_LONG(REG, LDSC)                                                                                     \
+    do {                                                                                                           \
+        auto kern = ce_forward_long_kernel<T, REG, LDSC>;                                                          \
+        const size_t lds = (size_t)(LDSC) * kLongThreads * sizeof(u32x4);                                          \
+        static const hipError_t attr = hipFuncSetAttribute((const void *)kern,                                     \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);  \
+        if (attr != hipSuccess) return fail((int)attr, who, attr);                                                 \
+        hipLaunchKernelGGL(kern, dim3((unsigned)m), dim3(kLongThreads), lds, s, n, nvec, (const uint16_t *)input,  \
+                           (const int32_t *)target, (uint16_t *)softmax, (float *)output, ignore_index);           \
+    } while (0)
+
+template <typename T>
+static int ce_forward(int32_t m, int32_t n, const void *input, const void *target, void *softmax, void *output,
+                      int32_t ignore_index, void *stream, const char *who) {
+    if (m <= 0 || n <= 0) return 0;
+    if (!input || !target || !softmax || !output) return fail(-1, "cross_entropy_forward launcher: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    const int32_t nvec = n / 8;
+    static const int force_sweep = env_int("BMT_CE_FORCE_SWEEP", 0);
+    if (!force_sweep && rows_vectorisable(n, input, softmax) && nvec <= 1024 * 16) {
+        if (nvec <= 64) BMT_CE_ROW(64, 1, true);
+        else if (nvec <= 128) BMT_CE_ROW(64, 2, true);
+        else if (nvec <= 256) BMT_CE_ROW(64, 4, true);
+        else if (nvec <= 512) BMT_CE_ROW(256, 2, true);
+        else if (nvec <= 1024) BMT_CE_ROW(256, 4, true);
+        else if (nvec <= 2048) BMT_CE_ROW(1024, 2, true);
+        else if (nvec <= 4096) BMT_CE_ROW(1024, 4, true);
+        else if (nvec <= 8192) BMT_CE_ROW(1024, 8, true);
+        else if (nvec <= 12288) BMT_CE_LONG(8, 4);
+        else BMT_CE_LONG(8, 8);
+    } else {
+        hipLaunchKernelGGL((ce_forward_sweep_kernel<T>), dim3((unsigned)m), dim3(kSweepThreads), 0, s, n,
+                           (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,
+                           ignore_index);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : fail((int)e, who, e);
+}
+
+template <typename T, int OP>
+static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void *row_b, const void *target, void *stream,
+                   const char *who) {
+    if (m <= 0 || n <= 0) return 0;
+    if (!x || !row_a || (OP == 1 && !row_b) || (OP == 0 && !target)) return fail(-1, "cross_entropy launcher: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (rows_vectorisable(n, x)) {
+        const int32_t nvec = n / 8;
+        const int64_t total = (int64_t)m * nvec;
+        hipLaunchKernelGGL((ce_flat_vec_kernel<T, OP>), dim3(flat_grid(total, kFlatThreads * kFlatUnroll)), dim3(kFlatThreads),
+                           0, s, nvec, total, (uint16_t *)x, (const float *)row_a, (const float *)row_b,
+                           (const int32_t *)target);
+    } else {
+        const int64_t total = (int64_t)m * n;
+        hipLaunchKernelGGL((ce_flat_scalar_kernel<T, OP>), dim3(flat_grid(total, kFlatThreads)), dim3(kFlatThreads), 0, s, n,
+                           total, (uint16_t *)x, (const float *)row_a, (const float *)row_b, (const int32_t *)target);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : fail((int)e, who, e);
+}
+
+template <typename T>
+static int sumexp(int32_t m, int32_t n, const void *logits, const void *row_max, void *row_sum, void *stream,
+                  const char *who) {
+    if (m <= 0 || n <= 0) return 0;
+    if (!logits || !row_max || !row_sum) return fail(-1, "fused_sumexp launcher: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (rows_vectorisable(n, logits))
+        hipLaunchKernelGGL((sumexp_kernel<T, true>), dim3((unsigned)m), dim3(kSweepThreads), 0, s, n, (const uint16_t *)logits,
+                           (const float *)row_max, (float *)row_sum);
+    else
+        hipLaunchKernelGGL((sumexp_kernel<T, false>), dim3((unsigned)m), dim3(kSweepThreads), 0, s, n, (const uint16_t *)logits,
+                           (const float *)row_max, (float *)row_sum);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : fail((int)e, who, e);
+}
+
+}  // namespace bmt
+
+using namespace bmt;
+
+extern "C" int cross_entropy_forward_fp16_launcher(int32_t m, int32_t n, const void *input, const void *target,
+                                                   void *softmax, void *output, int32_t ignore_index, void *stream) {
+    return ce_forward<Half>(m, n, input, target, softmax, output, ignore_index, stream, "cross_entropy_forward_fp16_launcher");
+}
+extern "C" int cross_entropy_forward_bf16_launcher(int32_t m, int32_t n, const void *input, const void *target,
+                                                   void *softmax, void *output, int32_t ignore_index, void *stream) {
+    return ce_forward<BFloat16>(m, n, input, target, softmax, output, ignore_index, stream, "cross_entropy_forward_bf16_launcher");
+}
+extern "C" int cross_entropy_backward_inplace_fp16_launcher(int32_t m, int32_t n, const void *grad_output,
+                                                            const void *target, void *x, int32_t ignore_index,
+                                                            void *stream) {
+    (void)ignore_index;  // cross_entropy.cu:46-60 never reads it
+    return ce_flat<Half, 0>(m, n, x, grad_output, nullptr, target, stream, "cross_entropy_backward_inplace_fp16_launcher");
+}
+extern "C" int cross_entropy_backward_inplace_bf16_launcher(int32_t m, int32_t n, const void *grad_output,
+                                                            const void *target, void *x, int32_t ignore_index,
+                                                            void *stream) {
+    (void)ignore_index;
+    return ce_flat<BFloat16, 0>(m, n, x, grad_output, nullptr, target, stream, "cross_entropy_backward_inplace_bf16_launcher");
+}
+extern "C" int fused_sumexp_fp16_launcher(int32_t m, int32_t n, const void *logits, const void *max_logits,
+                                          void *sum_exp_logits, void *stream) {
+    return sumexp<Half>(m, n, logits, max_logits, sum_exp_logits, stream, "fused_sumexp_fp16_launcher");
+}
+extern "C" int fused_sumexp_bf16_launcher(int32_t m, int32_t n, const void *logits, const void *max_logits,
+                                          void *sum_exp_logits, void *stream) {
+    return sumexp<BFloat16>(m, n, logits, max_logits, sum_exp_logits, stream, "fused_sumexp_bf16_launcher");
+}
+extern "C" int fused_softmax_inplace_fp16_launcher(int32_t m, int32_t n, void *logits, const void *max_logits,
+                                                   const void *sum_exp_logits, void *stream) {
+    return ce_flat<Half, 1>(m, n, logits, max_logits, sum_exp_logits, nullptr, stream, "fused_softmax_inplace_fp16_launcher");
+}
+extern "C" int fused_softmax_inplace_bf16_launcher(int32_t m, int32_t n, void *logits, const void *max_logits,
+                                                   const void *sum_exp_logits, void *stream) {
+    return ce_flat<BFloat16, 1>(m, n, logits, max_logits, sum_exp_logits, nullptr, stream, "fused_softmax_inplace_bf16_launcher");
+}

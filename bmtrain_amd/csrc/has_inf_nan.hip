@@ -1,0 +1,104 @@
+// Loss-scale overflow check for gfx950: does a 16-bit float buffer hold an inf or NaN?
+// Replaces csrc/cuda/has_inf_nan.cu:35-138 of the reference (two kernels and a
+// 1024-byte intermediate) by one streaming kernel.
+//
+// An element is inf/NaN iff its exponent field is all ones.  Two elements are
+// tested per dword without unpacking: mask the exponent fields and add the value
+// that makes an all-ones field carry into bit 15 of its half; no other field value
+// reaches bit 15, and the mask keeps the low half's carry out of the high half:
+//     hit |= ((w & EXP_MASK2) + EXP_CARRY2) & 0x80008000
+// Each lane ORs its dwords, the wave votes with one ballot, the waves of a
+// workgroup meet in one LDS word, and one lane per workgroup that saw a hit issues
+// a single relaxed atomic byte store out[0] = 1.  When nothing is found the
+// kernel writes nothing, which keeps the flag sticky across calls.
+#include "bmt_device.h"
+#include "bmt_host.h"
+#include "../../include/bmt_hip.h"
+
+namespace bmt {
+
+constexpr int kScanThreads = 256;
+
+template <typename T>
+__device__ __forceinline__ uint32_t exp_all_ones2(uint32_t w) {
+    return ((w & T::kExpMask2) + T::kExpCarry2) & 0x80008000u;
+}
+
+template <typename T, int UNROLL>
+__global__ __launch_bounds__(kScanThreads) void has_inf_nan_kernel(
+    const uint16_t *__restrict__ g, int64_t head, int64_t nvec, int64_t n, uint8_t *__restrict__ out) {
+    uint32_t hit = 0;
+    const u32x4 *body = (const u32x4 *)(g + head);
+    const int64_t tile = (int64_t)kScanThreads * UNROLL;
+    const int64_t ntiles = (nvec + tile - 1) / tile;
+    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const int64_t base = t * tile + threadIdx.x;
+        if (t * tile + tile <= nvec) {
+            u32x4 w[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) w[u] = __builtin_nontemporal_load(body + base + (int64_t)u * kScanThreads);
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++)
+                hit |= exp_all_ones2<T>(w[u].x) | exp_all_ones2<T>(w[u].y) | exp_all_ones2<T>(w[u].z) |
+                       exp_all_ones2<T>(w[u].w);
+        } else {
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const int64_t i = base + (int64_t)u * kScanThreads;
+                if (i < nvec) {
+                    u32x4 w = __builtin_nontemporal_load(body + i);
+                    hit |= exp_all_ones2<T>(w.x) | exp_all_ones2<T>(w.y) | exp_all_ones2<T>(w.z) | exp_all_ones2<T>(w.w);
+                }
+            }
+        }
+    }
+    // Unaligned head (< 8 elements) and tail (< 8 elements): workgroup 0, one element per lane.
+    if (blockIdx.x == 0) {
+        const int64_t tail_lo = head + nvec * 8;
+        const int64_t edge = head + (n - tail_lo);
+        if ((int64_t)threadIdx.x < edge) {
+            const int64_t i = (int64_t)threadIdx.x < head ? (int64_t)threadIdx.x : tail_lo + ((int64_t)threadIdx.x - head);
+            hit |= exp_all_ones2<T>((uint32_t)g[i]);
+        }
+    }
+    __shared__ uint32_t any_wave;
+    if (threadIdx.x == 0) any_wave = 0;
+    __syncthreads();
+    const bool wave_hit = __builtin_amdgcn_ballot_w64(hit != 0) != 0;
+    if (wave_hit && (threadIdx.x & (kWave - 1)) == 0) any_wave = 1;
+    __syncthreads();
+    if (threadIdx.x == 0 && any_wave)
+        __hip_atomic_store(out, (uint8_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <typename T>
+static int scan(int64_t n, const void *g, void *out, void *stream, const char *who) {
+    if (n <= 0) return 0;  // has_inf_nan.cu:108,:128
+    if (!g || !out) return fail(-1, "has_nan_inf launcher: null pointer");
+    const uintptr_t a = (uintptr_t)g;
+    if (a & 1u) return fail(-1, "has_nan_inf launcher: gradient pointer is not 2-byte aligned");
+    int64_t head = (int64_t)(((16 - (a & 15u)) & 15u) / 2);
+    if (head > n) head = n;
+    const int64_t nvec = (n - head) / 8;
+    constexpr int UNROLL = 4;
+    const int64_t tile = (int64_t)kScanThreads * UNROLL;
+    const int64_t ntiles = (nvec + tile - 1) / tile;
+    static const int per_cu = env_int("BMT_SCAN_BLOCKS_PER_CU", 8);
+    const int64_t cap = (int64_t)device_cu_count() * per_cu;
+    const int64_t grid = ntiles < 1 ? 1 : (ntiles < cap ? ntiles : cap);
+    hipLaunchKernelGGL((has_inf_nan_kernel<T, UNROLL>), dim3((unsigned)grid), dim3(kScanThreads), 0, (hipStream_t)stream,
+                       (const uint16_t *)g, head, nvec, n, (uint8_t *)out);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : fail((int)e, who, e);
+}
+
+}  // namespace bmt
+
+extern "C" int has_nan_inf_fp16_launcher(int64_t n, const void *g_fp16, void *mid, void *out, void *stream) {
+    (void)mid;
+    return bmt::scan<bmt::Half>(n, g_fp16, out, stream, "has_nan_inf_fp16_launcher");
+}
+extern "C" int has_nan_inf_bf16_launcher(int64_t n, const void *g_bf16, void *mid, void *out, void *stream) {
+    (void)mid;
+    return bmt::scan<bmt::BFloat16>(n, g_bf16, out, stream, "has_nan_inf_bf16_launcher");
+}

@@ -1,0 +1,106 @@
+"""Fused cross-entropy — API of bmtrain/loss/cross_entropy.py (non-parallel part).
+
+``OpFusedCrossEntropy`` runs the forward kernel (softmax into a scratch tensor plus the
+per-row loss) and, in backward, turns that same scratch tensor into the logits gradient
+in place and returns it.  ``FusedCrossEntropy`` adds what torch.nn.CrossEntropyLoss
+offers around it: ``ignore_index``, class weights, ``none`` / ``sum`` / ``mean``.
+"""
+from typing import Optional
+
+import torch
+
+from . import _function as F
+
+
+class OpFusedCrossEntropy(torch.autograd.Function):
+    """Cross-entropy over dim 1 of a 16-bit [N, C] tensor; returns the fp32 loss per row."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, target: torch.Tensor, ignore_index: int):
+        assert x.ndim == 2
+        x = x.contiguous()
+        target = target.contiguous()
+        softmax = torch.empty(x.size(), device=x.device, dtype=x.dtype)
+        out = torch.empty(x.size(0), device=x.device, dtype=torch.float)
+        F.cross_entropy_forward(x.size(0), x.size(1), x, target, softmax, out, ignore_index)
+        ctx.ignore_index = ignore_index
+        ctx.save_for_backward(softmax, target)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        grad_output = grad_output.contiguous()
+        softmax, target = ctx.saved_tensors
+        F.cross_entropy_backward_inplace(softmax.size(0), softmax.size(1), grad_output, target, softmax,
+                                         ctx.ignore_index)
+        return (softmax, None, None)
+
+
+class FusedCrossEntropy(torch.nn.Module):
+    r"""Cross entropy between raw scores ``input`` of shape :math:`(N, C)` and class indices
+    ``target`` of shape :math:`(N)`, like :class:`torch.nn.CrossEntropyLoss`:
+
+    .. math::
+        l_n = - w_{y_n} \log \frac{\exp(x_{n,y_n})}{\sum_{c} \exp(x_{n,c})} \cdot 1\{y_n \ne \text{ignore\_index}\}
+
+    reduced by ``reduction``: ``'none'``, ``'sum'``, or ``'mean'`` (the sum divided by
+    :math:`\sum_n w_{y_n} 1\{y_n \ne \text{ignore\_index}\}`).
+
+    fp32 input is handed to ``torch.nn.functional.cross_entropy`` (the only path that honours
+    ``label_smoothing``); fp16 / bf16 input takes the fused kernels.
+
+    Args:
+        weight: optional 1-D tensor of ``C`` class weights.
+        ignore_index: target value that contributes neither loss nor gradient.
+        reduction: ``'none'`` | ``'mean'`` | ``'sum'``.
+        label_smoothing: only applied to fp32 input.
+        parallel: vocabulary-parallel loss across tensor-parallel ranks; needs the
+            distributed runtime and is not available in this single-GPU package.
+
+    Example::
+
+        >>> loss_func = bmtrain_amd.loss.FusedCrossEntropy()
+        >>> logits = torch.randn(32, 100, device="cuda").half().requires_grad_()
+        >>> target = torch.randint(0, 100, (32,), device="cuda")
+        >>> loss_func(logits, target).backward()
+    """
+
+    def __init__(self, weight: Optional[torch.Tensor] = None, ignore_index: int = -100, reduction: str = "mean",
+                 label_smoothing: float = 0.0, parallel: bool = False) -> None:
+        super().__init__()
+        self.weight = weight
+        self.ignore_index = ignore_index
+        self.reduction = reduction
+        self.label_smoothing = label_smoothing
+        self.parallel = parallel
+
+    def forward(self, input: torch.Tensor, target: torch.Tensor) -> torch.Tensor:
+        if self.parallel:
+            raise NotImplementedError(
+                "FusedCrossEntropy(parallel=True) needs tensor-parallel all-reduces, which this "
+                "single-GPU package does not provide"
+            )
+        if input.dtype == torch.float32:
+            return torch.nn.functional.cross_entropy(
+                input, target.long(), weight=self.weight, ignore_index=self.ignore_index,
+                reduction=self.reduction, label_smoothing=self.label_smoothing)
+
+        ret = OpFusedCrossEntropy.apply(input, target.int(), self.ignore_index)
+
+        ignored = target == self.ignore_index
+        if self.weight is not None:
+            if self.weight.dim() != 1 or self.weight.size(0) != input.size(1):
+                raise ValueError("weight should be a 1D tensor of size C")
+            w = self.weight[torch.where(ignored, 0, target)].float()
+            w[ignored] = 0
+        else:
+            w = (~ignored).int()
+
+        ret = w * ret
+        if self.reduction == "none":
+            return ret
+        if self.reduction == "sum":
+            return ret.sum()
+        if self.reduction == "mean":
+            return ret.sum() / w.sum().float()
+        raise ValueError(f"{self.reduction} is not a valid value for reduction")

@@ -1,0 +1,121 @@
+"""Argument checking and dispatch in front of the Adam launchers.
+
+Same functions, argument order and failure modes as bmtrain/optim/_function.py:
+AssertionError for layout / dtype / device / size mismatches, NotImplementedError
+when bf16 is unavailable; the bias corrections are computed here in Python double
+(``1 - beta ** step``) and cross the C ABI as floats.
+"""
+import torch
+
+from .. import C
+
+_SIXTEEN_BIT = (torch.float16, torch.bfloat16)
+
+
+def _current_stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _on_gpu(t: torch.Tensor) -> bool:
+    return t.is_contiguous() and t.is_cuda
+
+
+def _same_numel(ref_name, ref, **others):
+    for name, t in others.items():
+        assert ref.numel() == t.numel(), f"{ref_name} and {name} must have the same number of elements"
+
+
+def _require_bf16():
+    if not C.is_bf16_supported():
+        raise NotImplementedError("bfloat16 is not supported on current GPU")
+
+
+def bf16_from_fp32(param_fp32: torch.Tensor) -> torch.Tensor:
+    """Host conversion by truncation (bmtrain/optim/_function.py:7-12)."""
+    out = torch.empty_like(param_fp32, dtype=torch.bfloat16)
+    C.to_bf16_from_fp32(param_fp32.numel(), param_fp32.data_ptr(), out.data_ptr())
+    return out
+
+
+def fp16_from_fp32(param_fp32: torch.Tensor) -> torch.Tensor:
+    """Host conversion, round to nearest even (bmtrain/optim/_function.py:15-20)."""
+    out = torch.empty_like(param_fp32, dtype=torch.float16)
+    C.to_fp16_from_fp32(param_fp32.numel(), param_fp32.data_ptr(), out.data_ptr())
+    return out
+
+
+def adam_cpu(param_fp32, param_fp16, delta_info, g_fp16, m_fp32, v_fp32,
+             beta1: float, beta2: float, eps: float, lr: float, scale: float, weight_decay: float, step: int) -> None:
+    """Host-memory Adam step (bmtrain/optim/_function.py:23-100)."""
+    cpu = torch.device("cpu")
+    named = dict(param_fp32=param_fp32, param_fp16=param_fp16, g_fp16=g_fp16, m_fp32=m_fp32, v_fp32=v_fp32)
+    for name, t in named.items():
+        assert t.is_contiguous(), f"{name} must be contiguous"
+    for name in ("param_fp32", "m_fp32", "v_fp32"):
+        assert named[name].dtype == torch.float32, f"{name} must be float32 tensor"
+    for name in ("param_fp16", "g_fp16"):
+        assert named[name].dtype in _SIXTEEN_BIT, f"{name} must be float16/bfloat16 tensor"
+    for name, t in named.items():
+        assert t.device == cpu, f"{name} must be a cpu tensor"
+    _same_numel("param_fp32", param_fp32, param_fp16=param_fp16, g_fp16=g_fp16, m_fp32=m_fp32, v_fp32=v_fp32)
+    if delta_info is not None:
+        assert delta_info.is_contiguous(), "delta_info must be contiguous"
+        assert delta_info.dtype == torch.float32, "delta_info must be float32 tensor"
+        assert delta_info.device == cpu, "delta_info must be a cpu tensor"
+        assert delta_info.numel() == 4, "delta_info have a length of 4"
+    bias_correction1 = 1 - beta1 ** step
+    bias_correction2 = 1 - beta2 ** step
+    if g_fp16.dtype == torch.bfloat16:
+        _require_bf16()
+        launcher = C.adam_cpu_bf16_launcher
+    else:
+        launcher = C.adam_cpu_fp16_launcher
+    launcher(
+        param_fp32.numel(), param_fp32.data_ptr(), param_fp16.data_ptr(),
+        delta_info.data_ptr() if delta_info is not None else 0,
+        g_fp16.data_ptr(), m_fp32.data_ptr(), v_fp32.data_ptr(),
+        beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2,
+    )
+
+
+def adam_fp16(param_fp32, param_fp16, g_fp16, m_fp16, v_fp32,
+              beta1: float, beta2: float, eps: float, lr: float, scale: float, weight_decay: float, step: int) -> None:
+    """Fused GPU step, fp16 parameters: moments live multiplied by ``scale``
+    (bmtrain/optim/_function.py:103-158)."""
+    named = dict(param_fp32=param_fp32, param_fp16=param_fp16, g_fp16=g_fp16, m_fp16=m_fp16, v_fp32=v_fp32)
+    for name, t in named.items():
+        assert _on_gpu(t), f"{name} must be contiguous and on cuda"
+    for name in ("param_fp32", "v_fp32"):
+        assert named[name].dtype == torch.float32, f"{name} must be float32 tensor"
+    for name in ("param_fp16", "g_fp16", "m_fp16"):
+        assert named[name].dtype == torch.float16, f"{name} must be float16 tensor"
+    _same_numel("param_fp32", param_fp32, param_fp16=param_fp16, g_fp16=g_fp16, m_fp16=m_fp16, v_fp32=v_fp32)
+    bias_correction1 = 1 - beta1 ** step
+    bias_correction2 = 1 - beta2 ** step
+    C.adam_fp16_launcher(
+        param_fp32.numel(), param_fp32.data_ptr(), param_fp16.data_ptr(), g_fp16.data_ptr(),
+        m_fp16.data_ptr(), v_fp32.data_ptr(),
+        beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2, _current_stream(),
+    )
+
+
+def adam_bf16(param_fp32, param_bf16, g_bf16, m_fp32, v_fp32,
+              beta1: float, beta2: float, eps: float, lr: float, scale: float, weight_decay: float, step: int) -> None:
+    """Fused GPU step, bf16 parameters: gradient is unscaled, moments are plain fp32
+    (bmtrain/optim/_function.py:161-218)."""
+    named = dict(param_fp32=param_fp32, param_bf16=param_bf16, g_bf16=g_bf16, m_fp32=m_fp32, v_fp32=v_fp32)
+    for name, t in named.items():
+        assert _on_gpu(t), f"{name} must be contiguous and on cuda"
+    for name in ("param_fp32", "m_fp32", "v_fp32"):
+        assert named[name].dtype == torch.float32, f"{name} must be float32 tensor"
+    for name in ("param_bf16", "g_bf16"):
+        assert named[name].dtype == torch.bfloat16, f"{name} must be bfloat16 tensor"
+    _same_numel("param_fp32", param_fp32, param_bf16=param_bf16, g_bf16=g_bf16, m_fp32=m_fp32, v_fp32=v_fp32)
+    bias_correction1 = 1 - beta1 ** step
+    bias_correction2 = 1 - beta2 ** step
+    _require_bf16()
+    C.adam_bf16_launcher(
+        param_fp32.numel(), param_fp32.data_ptr(), param_bf16.data_ptr(), g_bf16.data_ptr(),
+        m_fp32.data_ptr(), v_fp32.data_ptr(),
+        beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2, _current_stream(),
+    )

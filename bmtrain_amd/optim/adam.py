@@ -1,0 +1,116 @@
+"""On-device Adam for fp32 / fp16 / bf16 parameters — API of bmtrain/optim/adam.py.
+
+16-bit parameters take one fused HIP launch per tensor (``_function.adam_fp16`` /
+``adam_bf16``): fp32 master copy, moments and the 16-bit parameter are updated in a
+single pass over memory.  State layout per parameter (part of the checkpoint format):
+``step`` (int), ``exp_avg`` (fp16 for fp16 parameters, else fp32), ``exp_avg_sq``
+(fp32), ``_param_fp32`` (fp32 master, 16-bit parameters only).  For fp16 parameters
+the two moments are stored multiplied by the loss scale, which is why
+``_on_justify_scale`` rescales them whenever the scale changes.
+"""
+import torch
+
+from . import _function as F
+from ._base import check_grad, remap_loaded_state, torch_adam_fp32, validate_hyper, wants_maximize
+
+
+class AdamOptimizer(torch.optim.Optimizer):
+    """Adam optimizer support fp16 and bf16."""
+
+    _bmtrain_optimizer = True
+
+    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0, hold_steps=0):
+        validate_hyper(lr, betas, eps, weight_decay)
+        super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
+        self._hold_steps = hold_steps
+
+    def _on_justify_scale(self, old_scale, new_scale):
+        """fp16 moments are kept as moment * loss_scale (adam.py:46-55)."""
+        ratio = new_scale / old_scale
+        for group in self.param_groups:
+            for p in group["params"]:
+                state = self.state.get(p)
+                if state and p.dtype == torch.float16:
+                    state["exp_avg"] *= ratio
+                    state["exp_avg_sq"] *= ratio
+
+    def _init_state(self, p):
+        moment_dtype = torch.float16 if p.dtype == torch.float16 else torch.float32
+        state = self.state[p]
+        state["step"] = 0
+        state["exp_avg"] = torch.zeros(p.size(), dtype=moment_dtype, device=p.device)
+        state["exp_avg_sq"] = torch.zeros(p.size(), dtype=torch.float32, device=p.device)
+        if p.dtype != torch.float32:
+            state["_param_fp32"] = torch.empty(p.size(), dtype=torch.float32, device=p.device)
+            state["_param_fp32"].copy_(p)
+        return state
+
+    @torch.no_grad()
+    def step(self, closure=None, scale=1):
+        """One optimisation step; ``scale`` is the loss scale the gradients carry."""
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+
+        for group in self.param_groups:
+            beta1, beta2 = group["betas"][0], group["betas"][1]
+            for p in group["params"]:
+                if p.grad is None or not p.requires_grad:
+                    continue
+                check_grad(p)
+                state = self.state[p]
+                if len(state) == 0:
+                    state = self._init_state(p)
+                grad = -p.grad if wants_maximize(group) else p.grad
+
+                if p.dtype == torch.float32:
+                    # hold_steps is tested before the increment on this path (adam.py:137).
+                    lr = 0.0 if state["step"] < self._hold_steps else group["lr"]
+                    torch_adam_fp32(p, grad / scale, state["exp_avg"], state["exp_avg_sq"], state["step"],
+                                    beta1=beta1, beta2=beta2, lr=lr, weight_decay=group["weight_decay"],
+                                    eps=group["eps"])
+                    state["step"] += 1
+                else:
+                    # ... and after the increment on the fused path (adam.py:145,155).
+                    state["step"] += 1
+                    lr = 0.0 if state["step"] < self._hold_steps else group["lr"]
+                    fused = F.adam_fp16 if p.dtype == torch.float16 else F.adam_bf16
+                    fused(state["_param_fp32"], p, grad, state["exp_avg"], state["exp_avg_sq"],
+                          beta1, beta2, group["eps"], lr, scale, group["weight_decay"], state["step"])
+        return loss
+
+    def get_avg_delta():
+        raise NotImplementedError(
+            "get delta info is not supported in Adam optimizer , try bmt.optim.AdamOffloadOptimizer"
+        )
+
+    def get_var_delta():
+        raise NotImplementedError(
+            "get delta info is not supported in Adam optimizer , try bmt.optim.AdamOffloadOptimizer"
+        )
+
+    def load_state_dict(self, state_dict: dict) -> None:
+        """Loads optimizer state, casting each tensor to the dtype / device this optimizer
+        keeps it in and rebuilding a missing fp32 master copy from the parameter
+        (adam.py:175-248)."""
+
+        def convert(param, entry):
+            if param.dtype != torch.float32 and "_param_fp32" not in entry:
+                entry["_param_fp32"] = torch.empty(param.size(), dtype=torch.float32, device=param.device)
+                entry["_param_fp32"].copy_(param)
+            wanted = {
+                "exp_avg": torch.float16 if param.dtype == torch.float16 else torch.float32,
+                "exp_avg_sq": torch.float32,
+                "_param_fp32": torch.float32,
+            }
+            for name, dtype in wanted.items():
+                if name in entry:
+                    entry[name] = entry[name].to(param.device).to(dtype)
+            return entry
+
+        remap_loaded_state(self, state_dict, convert)
+
+    # zero_grad(set_to_none=True) breaks gradient accumulation into persistent buffers.
+    def zero_grad(self, set_to_none: bool = False):
+        super().zero_grad(set_to_none=set_to_none)

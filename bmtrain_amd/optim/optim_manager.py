@@ -1,0 +1,171 @@
+"""Loss scaling, overflow skip and optimizer stepping — API of
+bmtrain/optim/optim_manager.py, single GPU.
+
+The overflow check walks the 16-bit gradients with the ``has_inf_nan`` scan (one sticky
+flag for all tensors, one host read at the end).  Cross-rank reductions of the flag and
+of the gradient norm belong to the distributed runtime and are not performed here.
+"""
+from typing import Optional
+
+import torch
+
+from ..global_var import config
+from ..loss._function import has_inf_nan
+
+
+def check_overflow(param_groups):
+    """Raises OverflowError when any non-fp32 gradient holds an inf or NaN
+    (optim_manager.py:9-21)."""
+    flag = torch.zeros(1, dtype=torch.uint8, device="cuda")[0]
+    for group in param_groups:
+        for p in group["params"]:
+            if p.grad is not None and p.dtype != torch.float:
+                has_inf_nan(p.grad, flag)
+    if flag > 0:
+        raise OverflowError("Gradient overflow")
+
+
+def grad_rescale(param_groups, scale):
+    for group in param_groups:
+        for p in group["params"]:
+            if p.grad is not None and p.requires_grad:
+                p.grad /= scale
+
+
+class OptimManager:
+    """Steps a set of optimizers (and their lr schedulers) that share one dynamic loss scale.
+
+    >>> manager = OptimManager(loss_scale=1024)
+    >>> manager.add_optimizer(optimizer, lr_scheduler)
+    >>> manager.zero_grad(); manager.backward(loss); manager.step()
+    """
+
+    def __init__(self, loss_scale: Optional[float] = None, loss_scale_factor: float = 2,
+                 loss_scale_steps: int = 1024, min_loss_scale=1, max_loss_scale=float("inf"),
+                 grad_scale: Optional[int] = None):
+        self.loss_scale_enabled = loss_scale is not None
+        self.loss_scale = loss_scale if self.loss_scale_enabled else 1
+        self.steps_since_last_scale = 0
+        self.loss_scale_factor = loss_scale_factor if loss_scale_factor > 1 else 1 / loss_scale_factor
+        self.loss_scale_steps = loss_scale_steps
+        self.min_loss_scale = min_loss_scale
+        self.max_loss_scale = max_loss_scale
+        self.grad_scale = config["zero_size"] if grad_scale is None else grad_scale
+        self.optimizers = []
+        self.lr_schedulers = []
+
+    def add_optimizer(self, optimizer: torch.optim.Optimizer, lr_scheduler=None):
+        """All optimizers of one manager share the loss scale."""
+        self.optimizers.append(optimizer)
+        self.lr_schedulers.append(lr_scheduler)
+
+    def scale_loss(self, loss: torch.Tensor) -> torch.Tensor:
+        return loss * (self.loss_scale / self.grad_scale)
+
+    @staticmethod
+    def _join_load_stream(after_step: bool):
+        """Orders the compute stream against the runtime's copy stream when one is
+        registered (optim_manager.py:103-105, :155-156)."""
+        load_stream = config.get("load_stream")
+        if load_stream is None:
+            return
+        current = torch.cuda.current_stream()
+        if after_step:
+            load_stream.wait_stream(current)
+        else:
+            current.wait_stream(load_stream)
+
+    def backward(self, loss: torch.Tensor):
+        self.scale_loss(loss).backward()
+        self._join_load_stream(after_step=False)
+
+    def zero_grad(self):
+        for optimizer in self.optimizers:
+            optimizer.zero_grad(set_to_none=False)
+
+    def _overflowed(self) -> bool:
+        for optimizer in self.optimizers:
+            try:
+                check_overflow(optimizer.param_groups)
+            except OverflowError:
+                return True
+        return False
+
+    def step(self):
+        """Skips the step and lowers the scale on overflow; otherwise steps every optimizer
+        and scheduler and raises the scale after ``loss_scale_steps`` clean steps."""
+        if self.loss_scale_enabled and self._overflowed():
+            lowered = self.loss_scale / self.loss_scale_factor
+            print("Gradient overflow, change scale from %lf to %lf" % (self.loss_scale, lowered))
+            with torch.no_grad():
+                if self.loss_scale > self.min_loss_scale:
+                    self._justify_scale(lowered)
+                self.zero_grad()
+            return
+        for optimizer, lr_scheduler in zip(self.optimizers, self.lr_schedulers):
+            if getattr(optimizer, "_bmtrain_optimizer", False):
+                optimizer.step(scale=self.loss_scale)
+            else:
+                if self.loss_scale_enabled:
+                    grad_rescale(optimizer.param_groups, self.loss_scale)
+                optimizer.step()
+            if lr_scheduler is not None:
+                lr_scheduler.step()
+        if self.loss_scale_enabled:
+            self.steps_since_last_scale += 1
+            if self.steps_since_last_scale >= self.loss_scale_steps and self.loss_scale < self.max_loss_scale:
+                self._justify_scale(self.loss_scale * self.loss_scale_factor)
+        self._join_load_stream(after_step=True)
+
+    def clip_grad_norm(self, param_groups, max_norm, norm_type=2, eps=1e-6):
+        """Clips the (still loss-scaled) gradients to ``max_norm`` in place and returns the
+        unscaled total norm (optim_manager.py:158-200)."""
+        scale = self.loss_scale
+        parameters = [p for group in param_groups for p in group["params"]]
+        grads = [p.grad.data if p.grad is not None else torch.zeros_like(p.data) for p in parameters]
+        if norm_type == "inf":
+            total_norm = max(g.abs().max() for g in grads).detach()
+        else:
+            norm_type = float(norm_type)
+            acc = torch.zeros(1, dtype=torch.float32, device=grads[0].device if grads else "cuda")
+            for g in grads:
+                acc += g.float().norm(norm_type) ** norm_type
+            total_norm = acc[0] ** (1.0 / norm_type)
+        clip_coef = float(max_norm * scale) / (total_norm + eps)
+        if clip_coef < 1:
+            for p in parameters:
+                if p.grad is not None:
+                    p.grad.data.mul_(clip_coef)
+        return total_norm / scale
+
+    @torch.no_grad()
+    def _justify_scale(self, scale):
+        for optimizer in self.optimizers:
+            if hasattr(optimizer, "_on_justify_scale"):
+                optimizer._on_justify_scale(self.loss_scale, scale)
+        self.loss_scale = scale
+        self.steps_since_last_scale = 0
+
+    def state_dict(self, gather_opt=False) -> dict:
+        def opt_state(opt):
+            try:
+                return opt.state_dict(gather_opt)
+            except TypeError:  # optimizers whose state_dict() takes no argument
+                return opt.state_dict()
+        return {
+            "optimizers": [opt_state(opt) for opt in self.optimizers],
+            "lr_schedulers": [s.state_dict() if s else None for s in self.lr_schedulers],
+            "loss_scale": self.loss_scale,
+            "loss_scale_enabled": self.loss_scale_enabled,
+        }
+
+    def load_state_dict(self, state_dict: dict) -> None:
+        assert len(self.optimizers) == len(state_dict["optimizers"])
+        assert len(self.lr_schedulers) == len(state_dict["lr_schedulers"])
+        for opt, saved in zip(self.optimizers, state_dict["optimizers"]):
+            opt.load_state_dict(saved)
+        for scheduler, saved in zip(self.lr_schedulers, state_dict["lr_schedulers"]):
+            if scheduler is not None:
+                scheduler.load_state_dict(saved)
+        self.loss_scale = state_dict["loss_scale"]
+        self.loss_scale_enabled = state_dict["loss_scale_enabled"]

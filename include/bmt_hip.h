@@ -1,0 +1,146 @@
+/*
+ * C ABI of libbmt_hip.so — the MI355X (gfx950) replacement for the hot-path
+ * part of BMTrain's compiled extension `bmtrain.C`.
+ *
+ * Every entry point has the name and positional argument order of the function
+ * that the reference registers under `bmtrain.C` (csrc/bind.cpp:3-35, prototypes
+ * in csrc/include/bind.hpp:5-111 and csrc/include/adam_cpu.hpp), so that a
+ * binding layer can forward its arguments unchanged.  Differences, all supersets:
+ *   - element counts are int64_t (the reference takes int/int32_t for the GPU
+ *     launchers); flat buffers beyond 2^31 elements are supported;
+ *   - pointers are typed `void *` instead of std::uintptr_t integers;
+ *   - every function returns int: 0 on success, otherwise a hipError_t value
+ *     (GPU launchers) or -1 (invalid argument); the reference returns void and
+ *     never looks at the launch status.  bmt_hip_last_error() describes the last
+ *     failure of the calling thread.
+ *
+ * Ownership: the caller owns every buffer; the library allocates nothing, keeps
+ * no state between calls and retains no pointer.  GPU launchers are asynchronous
+ * on `stream` (a hipStream_t; NULL = the default stream) and never synchronise.
+ * Device pointers must belong to the device that is current at the call.
+ */
+#ifndef BMT_HIP_H
+#define BMT_HIP_H
+
+#include <stdint.h>
+
+/* The library is built with hidden visibility; only these entry points are exported. */
+#define BMT_API __attribute__((visibility("default")))
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* csrc/cuda/has_inf_nan.cu:140-145.  Always 1 on gfx950. */
+BMT_API int is_bf16_supported(void);
+
+/* Human-readable text for the last non-zero return value on this thread. */
+BMT_API const char *bmt_hip_last_error(void);
+
+/*
+ * has_nan_inf_{fp16,bf16}_launcher — csrc/cuda/has_inf_nan.cu:101-138 (bind.hpp:7-8).
+ * Sets out[0] = 1 (uint8) iff some g[i], 0 <= i < n, is +-inf or NaN; leaves out[0]
+ * untouched otherwise (the flag is sticky across calls).  n <= 0 is a no-op.
+ * `mid` is the reference's uint8[1024] scratch; it is accepted and not used.
+ */
+BMT_API int has_nan_inf_fp16_launcher(int64_t n, const void *g_fp16, void *mid, void *out, void *stream);
+BMT_API int has_nan_inf_bf16_launcher(int64_t n, const void *g_bf16, void *mid, void *out, void *stream);
+
+/*
+ * adam_fp16_launcher — csrc/cuda/adam_cuda.cu:76-101 (kernel :8-37; bind.hpp:82-96).
+ * One fused step over n elements.  fp16 flavour: g is the loss-scaled gradient and
+ * the moments are kept multiplied by `scale` (m in fp16, v in fp32).
+ * Writes param_fp32, param_fp16 (round-to-nearest-even), m_fp16, v_fp32.  n <= 0: no-op.
+ */
+BMT_API int adam_fp16_launcher(int64_t n, void *param_fp32, void *param_fp16, const void *g_fp16,
+                       void *m_fp16, void *v_fp32,
+                       float beta1, float beta2, float eps, float lr, float scale,
+                       float weight_decay, float bias_correction1, float bias_correction2,
+                       void *stream);
+
+/*
+ * adam_bf16_launcher — csrc/cuda/adam_cuda.cu:103-126 (kernel :39-72; bind.hpp:97-111).
+ * bf16 flavour: g is divided by `scale`; m and v are plain fp32 moments.
+ */
+BMT_API int adam_bf16_launcher(int64_t n, void *param_fp32, void *param_bf16, const void *g_bf16,
+                       void *m_fp32, void *v_fp32,
+                       float beta1, float beta2, float eps, float lr, float scale,
+                       float weight_decay, float bias_correction1, float bias_correction2,
+                       void *stream);
+
+/*
+ * adam_cpu_{fp16,bf16}_launcher — csrc/include/adam_cpu.hpp:504-533 and :535-557.
+ * Host-memory (optimizer-offload) Adam step; all pointers are host pointers.
+ * delta_info is NULL or float[4] receiving {mean, variance, sum, sum of squares} of the
+ * per-element update m/bc1/(sqrt(v/bc2)+eps) + wd*p.  The fp16 copy is rounded to
+ * nearest even, the bf16 copy is truncated, as in the reference.
+ */
+BMT_API int adam_cpu_fp16_launcher(int64_t n, void *param_fp32, void *param_fp16, void *delta_info,
+                           const void *g_fp16, void *m_fp32, void *v_fp32,
+                           float beta1, float beta2, float eps, float lr, float scale,
+                           float weight_decay, float bias_correction1, float bias_correction2);
+BMT_API int adam_cpu_bf16_launcher(int64_t n, void *param_fp32, void *param_bf16, void *delta_info,
+                           const void *g_bf16, void *m_fp32, void *v_fp32,
+                           float beta1, float beta2, float eps, float lr, float scale,
+                           float weight_decay, float bias_correction1, float bias_correction2);
+
+/*
+ * to_fp16_from_fp32 / to_bf16_from_fp32 — bind.cpp:4-5 ->
+ * fp16_from_fp32_value_launcher / bf16_from_fp32_value_launcher
+ * (csrc/include/adam_cpu.hpp:139-175).  Host pointers.  fp16: round to nearest even;
+ * bf16: truncation.
+ */
+BMT_API int to_fp16_from_fp32(int64_t n, const void *param_fp32, void *param_fp16);
+BMT_API int to_bf16_from_fp32(int64_t n, const void *param_fp32, void *param_bf16);
+
+/*
+ * cross_entropy_forward_{fp16,bf16}_launcher — csrc/cuda/cross_entropy.cu:202-217,
+ * :234-247 (kernels :9-43, :63-101; bind.hpp:20-28, :38-46).
+ * input, softmax: [m, n] row-major 16-bit; target: int32[m]; output: float[m].
+ *   softmax[r, :] = softmax(input[r, :]) rounded to the 16-bit type,
+ *   output[r]     = target[r] != ignore_index ? logsumexp(input[r, :]) - input[r, target[r]] : 0.
+ * m <= 0 or n <= 0 is a no-op (the reference would issue an invalid launch).
+ */
+BMT_API int cross_entropy_forward_fp16_launcher(int32_t m, int32_t n, const void *input, const void *target,
+                                        void *softmax, void *output, int32_t ignore_index, void *stream);
+BMT_API int cross_entropy_forward_bf16_launcher(int32_t m, int32_t n, const void *input, const void *target,
+                                        void *softmax, void *output, int32_t ignore_index, void *stream);
+
+/*
+ * cross_entropy_backward_inplace_{fp16,bf16}_launcher — csrc/cuda/cross_entropy.cu:219-232,
+ * :249-261 (kernels :46-60, :104-121; bind.hpp:29-37, :47-53).
+ * x holds the softmax written by the forward call and is overwritten with the gradient:
+ *   x[r, i] = to16((x[r, i] - (i == target[r])) * grad_output[r]).
+ * As in the reference, ignore_index is not consulted: ignored rows are zeroed by the caller
+ * passing grad_output[r] = 0.
+ */
+BMT_API int cross_entropy_backward_inplace_fp16_launcher(int32_t m, int32_t n, const void *grad_output,
+                                                 const void *target, void *x, int32_t ignore_index,
+                                                 void *stream);
+BMT_API int cross_entropy_backward_inplace_bf16_launcher(int32_t m, int32_t n, const void *grad_output,
+                                                 const void *target, void *x, int32_t ignore_index,
+                                                 void *stream);
+
+/*
+ * fused_sumexp_{fp16,bf16}_launcher — csrc/cuda/cross_entropy.cu:263-288 (kernels :124-164;
+ * bind.hpp:54-67).  sum_exp_logits[r] = sum_i expf(logits[r, i] - max_logits[r]).
+ */
+BMT_API int fused_sumexp_fp16_launcher(int32_t m, int32_t n, const void *logits, const void *max_logits,
+                               void *sum_exp_logits, void *stream);
+BMT_API int fused_sumexp_bf16_launcher(int32_t m, int32_t n, const void *logits, const void *max_logits,
+                               void *sum_exp_logits, void *stream);
+
+/*
+ * fused_softmax_inplace_{fp16,bf16}_launcher — csrc/cuda/cross_entropy.cu:290-315
+ * (kernels :167-199; bind.hpp:68-81).
+ * logits[r, i] = to16(expf(logits[r, i] - max_logits[r]) / sum_exp_logits[r]).
+ */
+BMT_API int fused_softmax_inplace_fp16_launcher(int32_t m, int32_t n, void *logits, const void *max_logits,
+                                        const void *sum_exp_logits, void *stream);
+BMT_API int fused_softmax_inplace_bf16_launcher(int32_t m, int32_t n, void *logits, const void *max_logits,
+                                        const void *sum_exp_logits, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BMT_HIP_H */
