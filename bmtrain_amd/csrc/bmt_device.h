@@ -19,6 +19,11 @@ struct Half {  // IEEE binary16
         return (float)__builtin_bit_cast(_Float16, b);          // exact, subnormals kept
     }
     static __device__ __forceinline__ uint16_t from_f32(float f) {
+        // The empty asm makes `f` exist as a rounded fp32 value.  Without it the compiler folds
+        // the multiply / fma that produced `f` into v_fma_mixlo_f16, which rounds the exact
+        // result once, straight to fp16, instead of to fp32 and then to fp16 as the reference
+        // arithmetic does; the two differ by one fp16 ulp near ties.
+        asm("" : "+v"(f));
         return __builtin_bit_cast(uint16_t, (_Float16)f);        // v_cvt_f16_f32, round-nearest-even
     }
     static constexpr uint32_t kExpMask2 = 0x7C007C00u;   // exponent field of both halves of a dword

@@ -39,7 +39,7 @@ def torch_adam_fp32(param, grad, exp_avg, exp_avg_sq, step, *, beta1, beta2, lr,
     adam_offload.py:156-187) they go through torch's functional Adam — coupled L2 decay,
     bias correction at ``step + 1`` — on whatever device the tensors live."""
     _torch_functional.adam(
-        [param], [grad], [exp_avg], [exp_avg_sq], [], [torch.tensor(step)],
+        [param], [grad], [exp_avg], [exp_avg_sq], [], [torch.tensor(float(step))],
         amsgrad=False, beta1=beta1, beta2=beta2, lr=lr, weight_decay=weight_decay, eps=eps, maximize=False,
     )
 

@@ -1,0 +1,269 @@
+"""Fused Adam on the GPU, through the C ABI, against the oracle.
+
+The kernels implement one fixed expression tree with correctly rounded division and square
+root, so the bar here is tighter than the stated tolerance (fp32 state <= 1e-6 relative,
+16-bit copy <= 1 ulp): every output must equal the oracle's bit for bit.  The oracle's tree is
+itself pinned to the reference's compiled CPU Adam (tests/test_oracle_adam.py)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from bmtrain_amd.optim import _function as F
+from conftest import bits16, f32_bits, from_bits16, load_golden
+
+pytestmark = pytest.mark.gpu
+HYP = dict(beta1=0.9, beta2=0.999, eps=1e-8, lr=1e-3, weight_decay=0.01)
+
+
+def _state(n, gen, flavour):
+    p = torch.randn(n, generator=gen) * 0.02
+    m = torch.randn(n, generator=gen) * 1e-4
+    v = (torch.randn(n, generator=gen) * 1e-6).abs()
+    if flavour == "fp16":
+        m = m.half()
+    return p, m, v
+
+
+def _run_both(flavour, p, m, v, g, scale, step, lr=HYP["lr"], wd=HYP["weight_decay"], offset=0):
+    """Steps GPU copies (placed `offset` elements into larger buffers) and oracle copies."""
+    dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
+    n = p.numel()
+
+    def place(t):
+        buf = torch.zeros(n + offset + 8, dtype=t.dtype, device="cuda")
+        buf[offset:offset + n] = t.cuda()
+        return buf, buf[offset:offset + n]
+
+    (pb, pg), (mb, mg), (vb, vg), (gb, gg) = place(p), place(m), place(v), place(g)
+    hb, hg = place(torch.zeros(n, dtype=dt16))
+    fn = F.adam_fp16 if flavour == "fp16" else F.adam_bf16
+    fn(pg, hg, gg, mg, vg, HYP["beta1"], HYP["beta2"], HYP["eps"], lr, scale, wd, step)
+    torch.cuda.synchronize()
+    # nothing outside the view may change
+    for buf in (pb, mb, vb, hb):
+        assert torch.count_nonzero(buf[:offset]) == 0 and torch.count_nonzero(buf[offset + n:]) == 0
+
+    po, vo, ho = p.numpy().copy(), v.numpy().copy(), np.zeros(n, np.uint16)
+    bc1, bc2 = oracle.bias_corrections(HYP["beta1"], HYP["beta2"], step)
+    if flavour == "fp16":
+        mo = bits16(m)
+        oracle.adam_gpu_fp16(po, ho, bits16(g), mo, vo, HYP["beta1"], HYP["beta2"], HYP["eps"], lr, scale, wd, bc1, bc2)
+        m_equal = np.array_equal(bits16(mg), mo)
+    else:
+        mo = m.numpy().copy()
+        oracle.adam_gpu_bf16(po, ho, bits16(g), mo, vo, HYP["beta1"], HYP["beta2"], HYP["eps"], lr, scale, wd, bc1, bc2)
+        m_equal = np.array_equal(f32_bits(mg.cpu().numpy()), f32_bits(mo))
+    assert np.array_equal(f32_bits(pg.cpu().numpy()), f32_bits(po)), "fp32 master"
+    assert np.array_equal(f32_bits(vg.cpu().numpy()), f32_bits(vo)), "second moment"
+    assert m_equal, "first moment"
+    assert np.array_equal(bits16(hg), ho), "16-bit copy"
+    return pg.cpu(), mg.cpu(), vg.cpu()
+
+
+@pytest.mark.parametrize("flavour", ["bf16", "fp16"])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 8, 63, 1023, 1024, 1025, 2047, 2048, 2049, 4099, (1 << 20) + 3])
+def test_bit_exact_against_oracle(flavour, n):
+    gen = torch.Generator().manual_seed(n)
+    dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
+    p, m, v = _state(n, gen, flavour)
+    for step, scale in ((1, 1.0), (2, 1024.0), (100, 3.0)):
+        g = (torch.randn(n, generator=gen) * 1e-3 * scale).to(dt16)
+        p, m, v = _run_both(flavour, p, m, v, g, scale, step)
+
+
+@pytest.mark.parametrize("flavour", ["bf16", "fp16"])
+@pytest.mark.parametrize("offset", [1, 2, 3, 4, 5, 6, 7])
+def test_views_at_any_element_offset(flavour, offset):
+    """Parameters are often slices of one flat buffer.  All arrays offset alike: vector body with
+    scalar head/tail; the guard elements around the views must stay untouched."""
+    gen = torch.Generator().manual_seed(offset)
+    dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
+    for n in (1, 3, 6, 1000, 5001):
+        p, m, v = _state(n, gen, flavour)
+        g = (torch.randn(n, generator=gen) * 1e-3).to(dt16)
+        _run_both(flavour, p, m, v, g, 1.0, 3, offset=offset)
+
+
+@pytest.mark.parametrize("flavour", ["bf16", "fp16"])
+def test_arrays_with_different_alignment_phases(flavour):
+    """fp32 master at offset 1, gradient at offset 2, ...: no common vector phase, element path."""
+    gen = torch.Generator().manual_seed(77)
+    dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
+    n = 3001
+    p, m, v = _state(n, gen, flavour)
+    g = (torch.randn(n, generator=gen) * 1e-3).to(dt16)
+    bufs = {}
+    for k, (name, t) in enumerate((("p", p), ("m", m), ("v", v), ("g", g), ("h", torch.zeros(n, dtype=dt16)))):
+        b = torch.zeros(n + 16, dtype=t.dtype, device="cuda")
+        b[k + 1:k + 1 + n] = t.cuda()
+        bufs[name] = b[k + 1:k + 1 + n]
+    fn = F.adam_fp16 if flavour == "fp16" else F.adam_bf16
+    fn(bufs["p"], bufs["h"], bufs["g"], bufs["m"], bufs["v"], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 5)
+    po, vo, ho = p.numpy().copy(), v.numpy().copy(), np.zeros(n, np.uint16)
+    bc1, bc2 = oracle.bias_corrections(0.9, 0.999, 5)
+    if flavour == "fp16":
+        mo = bits16(m)
+        oracle.adam_gpu_fp16(po, ho, bits16(g), mo, vo, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, bc1, bc2)
+    else:
+        mo = m.numpy().copy()
+        oracle.adam_gpu_bf16(po, ho, bits16(g), mo, vo, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, bc1, bc2)
+    assert np.array_equal(f32_bits(bufs["p"].cpu().numpy()), f32_bits(po))
+    assert np.array_equal(bits16(bufs["h"]), ho)
+
+
+def test_bf16_kernel_reproduces_the_reference_compiled_cpu_adam():
+    """Vectors written by the reference's own adam_cpu.hpp (bf16 path): the GPU kernel's fp32
+    parameters and moments are identical bit for bit; the bf16 copy is the round-to-nearest-even
+    neighbour of the reference CPU path's truncated copy (0 or 1 ulp above it)."""
+    g = load_golden("adam_cpu_bf16_t8")
+    n = int(g["n"])
+    p = torch.from_numpy(g["p0"].copy()).cuda()
+    m = torch.zeros(n, device="cuda"); v = torch.zeros(n, device="cuda")
+    h = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+    for s in range(1, int(g["steps"]) + 1):
+        grad = from_bits16(g[f"g{s}"], torch.bfloat16).cuda()
+        F.adam_bf16(p, h, grad, m, v, float(g["beta1"]), float(g["beta2"]), float(g["eps"]), float(g["lr"]),
+                    float(g["scale"]), float(g["weight_decay"]), s)
+        assert np.array_equal(f32_bits(p.cpu().numpy()), f32_bits(g[f"p{s}"]))
+        assert np.array_equal(f32_bits(m.cpu().numpy()), f32_bits(g[f"m{s}"]))
+        assert np.array_equal(f32_bits(v.cpu().numpy()), f32_bits(g[f"v{s}"]))
+        d = bits16(h).astype(np.int32) - g[f"h{s}"].astype(np.int32)
+        assert d.min() >= 0 and d.max() <= 1
+
+
+@pytest.mark.parametrize("flavour", ["bf16", "fp16"])
+def test_tolerances_against_float64(flavour):
+    """The stated bars, against a float64 evaluation: fp32 state <= 1e-6 relative (norm-wise),
+    16-bit copy <= 1 ulp of the float64 result."""
+    from conftest import ulp_distance16
+    gen = torch.Generator().manual_seed(21)
+    n = 200000
+    dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
+    scale = 1024.0 if flavour == "fp16" else 1.0
+    p = torch.randn(n, generator=gen) * 0.02
+    m_real = torch.randn(n, generator=gen) * 1e-4
+    v_real = (torch.randn(n, generator=gen) * 1e-6).abs()
+    g = (torch.randn(n, generator=gen) * 1e-3 * scale).to(dt16)
+    step = 100
+    pg, vg, gg = p.cuda(), (v_real * scale).cuda() if flavour == "fp16" else v_real.cuda(), g.cuda()
+    hg = torch.zeros(n, dtype=dt16, device="cuda")
+    if flavour == "fp16":
+        mg = (m_real * scale).half().cuda()
+        m_in = mg.double().cpu() / scale
+        F.adam_fp16(pg, hg, gg, mg, vg, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, step)
+    else:
+        mg = m_real.cuda()
+        m_in = m_real.double()
+        F.adam_bf16(pg, hg, gg, mg, vg, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, step)
+    f = lambda x: float(np.float32(x))
+    b1, b2, eps, lr, wd = f(0.9), f(0.999), f(1e-8), f(1e-3), f(0.01)
+    bc1, bc2 = (f(c) for c in oracle.bias_corrections(0.9, 0.999, step))
+    greal = g.double() / scale
+    m64 = b1 * m_in + f(np.float32(1) - np.float32(0.9)) * greal
+    v64 = b2 * v_real.double() + f(np.float32(1) - np.float32(0.999)) * greal * greal
+    p64 = p.double() - lr * (m64 / bc1) / (torch.sqrt(v64 / bc2) + eps) - lr * wd * p.double()
+    rel = lambda a, b: ((a - b).abs().max() / b.abs().max()).item()
+    assert rel(pg.double().cpu(), p64) <= 1e-6
+    assert rel(vg.double().cpu() / (scale if flavour == "fp16" else 1.0), v64) <= 1e-6
+    if flavour == "bf16":
+        assert rel(mg.double().cpu(), m64) <= 1e-6
+    assert ulp_distance16(bits16(hg), bits16(p64.to(dt16))).max() <= 1
+
+
+def test_lr_zero_holds_parameters():
+    n = 10000
+    gen = torch.Generator().manual_seed(8)
+    p = (torch.randn(n, generator=gen) * 0.02).cuda()
+    p0 = p.clone()
+    h = p.bfloat16()
+    m = torch.zeros(n, device="cuda"); v = torch.zeros(n, device="cuda")
+    g = torch.randn(n, generator=gen).bfloat16().cuda()
+    F.adam_bf16(p, h, g, m, v, 0.9, 0.999, 1e-8, 0.0, 1.0, 0.01, 1)
+    assert torch.equal(p, p0) and torch.count_nonzero(m) == n and torch.count_nonzero(v) == n
+
+
+def test_argument_checks():
+    n = 16
+    p = torch.zeros(n, device="cuda"); m = torch.zeros(n, device="cuda"); v = torch.zeros(n, device="cuda")
+    h = torch.zeros(n, dtype=torch.bfloat16, device="cuda"); g = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+    a = (0.9, 0.999, 1e-8, 1e-3, 1.0, 0.0, 1)
+    with pytest.raises(AssertionError, match="same number"):
+        F.adam_bf16(p, h, g[:8], m, v, *a)
+    with pytest.raises(AssertionError, match="bfloat16"):
+        F.adam_bf16(p, h.half(), g, m, v, *a)
+    with pytest.raises(AssertionError, match="cuda"):
+        F.adam_bf16(p.cpu(), h, g, m, v, *a)
+    with pytest.raises(AssertionError, match="float16"):
+        F.adam_fp16(p, h, g, m.half(), v, *a)
+
+
+def _fill_(x, std, gen, absolute=False, chunk=1 << 27):
+    for lo in range(0, x.numel(), chunk):
+        part = x[lo:lo + chunk]
+        r = torch.randn(part.numel(), generator=gen, device="cuda", dtype=torch.float32).mul_(std)
+        part.copy_(r.abs_() if absolute else r)
+
+
+def _check_slices(n, slices, before, after, step, scale):
+    bc1, bc2 = oracle.bias_corrections(0.9, 0.999, step)
+    for lo, hi in slices:
+        po, mo, vo = (before[k][lo:hi].cpu().numpy().copy() for k in ("p", "m", "v"))
+        ho = np.zeros(hi - lo, np.uint16)
+        oracle.adam_gpu_bf16(po, ho, bits16(before["g"][lo:hi]), mo, vo, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, bc1, bc2)
+        assert np.array_equal(f32_bits(after["p"][lo:hi].cpu().numpy()), f32_bits(po)), (lo, hi)
+        assert np.array_equal(f32_bits(after["m"][lo:hi].cpu().numpy()), f32_bits(mo)), (lo, hi)
+        assert np.array_equal(f32_bits(after["v"][lo:hi].cpu().numpy()), f32_bits(vo)), (lo, hi)
+        assert np.array_equal(bits16(after["h"][lo:hi]), ho), (lo, hi)
+
+
+def test_one_transformer_block_flat_buffer():
+    """202,383,360 elements (4*4096^2 + 3*4096*11008), step 100, scale 1.  Seeded slices are checked
+    against the oracle bit for bit; the whole buffer is checked by stepping a second copy in
+    three separately launched pieces (different tile-to-workgroup mapping) and comparing all of it."""
+    n = 202_383_360
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    before = {"p": torch.empty(n, device="cuda"), "m": torch.empty(n, device="cuda"), "v": torch.empty(n, device="cuda"),
+              "g": torch.empty(n, dtype=torch.bfloat16, device="cuda")}
+    _fill_(before["p"], 0.02, gen); _fill_(before["m"], 1e-4, gen); _fill_(before["v"], 1e-6, gen, absolute=True)
+    _fill_(before["g"], 1e-3, gen)
+    after = {k: before[k].clone() for k in ("p", "m", "v")}
+    after["h"] = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+    F.adam_bf16(after["p"], after["h"], before["g"], after["m"], after["v"], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100)
+    rnd = np.random.default_rng(1)
+    starts = [0, n - 70000] + [int(s) for s in rnd.integers(0, n - 70000, 6)]
+    _check_slices(n, [(s, s + 65536 + 11) for s in starts], before, after, 100, 1.0)
+    pieces = {k: before[k].clone() for k in ("p", "m", "v")}
+    pieces["h"] = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+    cuts = [0, 50_000_003, 120_000_001, n]
+    for lo, hi in zip(cuts[:-1], cuts[1:]):
+        F.adam_bf16(pieces["p"][lo:hi], pieces["h"][lo:hi], before["g"][lo:hi], pieces["m"][lo:hi], pieces["v"][lo:hi],
+                    0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100)
+    for k in ("p", "m", "v", "h"):
+        assert torch.equal(pieces[k].view(torch.int32 if k != "h" else torch.int16),
+                           after[k].view(torch.int32 if k != "h" else torch.int16)), k
+
+
+def test_more_than_2_to_the_31_elements():
+    """Element counts beyond int32 (the reference's launcher takes `int n`): the last stretch of a
+    2^31 + 12345 element buffer must be stepped, and stepped correctly."""
+    n = (1 << 31) + 12345
+    gen = torch.Generator(device="cuda").manual_seed(31)
+    before = {"p": torch.empty(n, device="cuda"), "m": torch.zeros(n, device="cuda"), "v": torch.zeros(n, device="cuda"),
+              "g": torch.empty(n, dtype=torch.bfloat16, device="cuda")}
+    _fill_(before["p"], 0.02, gen); _fill_(before["g"], 1e-3, gen)
+    slices = [(0, 4096), ((1 << 31) - 2048, (1 << 31) + 2048), (n - 12345, n)]
+    snap = {k: {s: before[k][s[0]:s[1]].clone() for s in slices} for k in ("p", "m", "v", "g")}
+    h = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+    F.adam_bf16(before["p"], h, before["g"], before["m"], before["v"], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 1)
+    bc1, bc2 = oracle.bias_corrections(0.9, 0.999, 1)
+    for s in slices:
+        po, mo, vo = (snap[k][s].cpu().numpy().copy() for k in ("p", "m", "v"))
+        ho = np.zeros(s[1] - s[0], np.uint16)
+        oracle.adam_gpu_bf16(po, ho, bits16(snap["g"][s]), mo, vo, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, bc1, bc2)
+        assert np.array_equal(f32_bits(before["p"][s[0]:s[1]].cpu().numpy()), f32_bits(po)), s
+        assert np.array_equal(f32_bits(before["v"][s[0]:s[1]].cpu().numpy()), f32_bits(vo)), s
+        assert np.array_equal(bits16(h[s[0]:s[1]]), ho), s
+    assert torch.count_nonzero(before["v"][-(1 << 20):]) == (1 << 20)
+    del before, h
+    torch.cuda.empty_cache()

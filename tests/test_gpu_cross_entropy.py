@@ -1,0 +1,306 @@
+"""Fused cross-entropy on the GPU, through the C ABI, against the oracle.
+
+Bars: loss <= 1e-3 relative to an fp32 reference (met with a wide margin: the test uses 2e-6);
+stored softmax and gradients <= 1 ulp of the 16-bit type against the oracle's restatement of the
+reference expressions.  The backward kernel alone is exact arithmetic on its 16-bit input, so
+on identical input it must match the oracle bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from bmtrain_amd.loss import _function as F
+from bmtrain_amd.loss import FusedCrossEntropy, OpFusedCrossEntropy
+from conftest import bits16, from_bits16, ulp_distance16
+
+pytestmark = pytest.mark.gpu
+DTYPES = [("fp16", torch.float16), ("bf16", torch.bfloat16)]
+
+
+def _case(m, n, dtype, seed, std=2.0, ignore_frac=0.1):
+    gen = torch.Generator().manual_seed(seed)
+    x = (torch.randn(m, n, generator=gen) * std).to(dtype)
+    t = torch.randint(0, n, (m,), generator=gen, dtype=torch.int32)
+    t[torch.rand(m, generator=gen) < ignore_frac] = -100
+    return x, t
+
+
+def _forward_gpu(x, t, ignore=-100):
+    xg, tg = x.cuda(), t.cuda()
+    softmax = torch.empty_like(xg)
+    out = torch.empty(x.size(0), dtype=torch.float32, device="cuda")
+    F.cross_entropy_forward(x.size(0), x.size(1), xg, tg, softmax, out, ignore)
+    return softmax, out
+
+
+# every launch shape of the forward: one wave per row, 256 and 1024 lanes per row with 1..8 vectors
+# per lane in registers, registers + LDS, and the element-load kernel (n % 8 != 0, or very long rows)
+WIDTHS = [1, 2, 3, 7, 8, 10, 16, 90, 100, 512, 520, 1000, 1024, 2048, 2056, 4096, 8192, 8200, 10240, 16384, 30000,
+          32000, 32768, 50264, 65536, 65544, 98304, 100000, 128256, 131072, 131080, 151936]
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+@pytest.mark.parametrize("n", WIDTHS)
+def test_forward_against_oracle(name, dtype, n):
+    m = 37 if n <= 4096 else 5
+    x, t = _case(m, n, dtype, seed=n)
+    softmax, loss = _forward_gpu(x, t)
+    want_soft, want_loss = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
+    assert ulp_distance16(bits16(softmax), want_soft).max() <= 1
+    assert (bits16(softmax) != want_soft).mean() < 0.01
+    np.testing.assert_allclose(loss.cpu().numpy(), want_loss, rtol=2e-6, atol=2e-6)
+    ref32 = torch.nn.functional.cross_entropy(x.float(), t.long(), ignore_index=-100, reduction="none").numpy()
+    np.testing.assert_allclose(loss.cpu().numpy(), ref32, rtol=1e-3, atol=1e-6)
+    assert np.all(loss.cpu().numpy()[t.numpy() == -100] == 0)
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+@pytest.mark.parametrize("n", [1, 5, 8, 100, 1000, 4096, 32000, 50001, 128256])
+def test_backward_bit_exact_on_identical_input(name, dtype, n):
+    m = 11
+    x, t = _case(m, n, dtype, seed=n + 1)
+    soft, _ = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
+    gen = torch.Generator().manual_seed(n)
+    for upstream in (1.0, 32768.0, 2.0 ** 20):
+        v = (torch.rand(m, generator=gen) * upstream / m).float()
+        v[t == -100] = 0
+        want = soft.copy()
+        oracle.ce_backward_inplace(v.numpy(), t.numpy(), want, -100, name)
+        xg = from_bits16(soft, dtype).reshape(m, n).cuda()
+        F.cross_entropy_backward_inplace(m, n, v.cuda(), t.cuda(), xg, -100)
+        assert np.array_equal(bits16(xg).reshape(m, n), want), upstream
+    # an ignored row with a non-zero grad_output is scaled, not zeroed (cross_entropy.cu:46-60)
+    v = torch.ones(m)
+    want = soft.copy()
+    oracle.ce_backward_inplace(v.numpy(), t.numpy(), want, -100, name)
+    xg = from_bits16(soft, dtype).reshape(m, n).cuda()
+    F.cross_entropy_backward_inplace(m, n, v.cuda(), t.cuda(), xg, -100)
+    assert np.array_equal(bits16(xg).reshape(m, n), want)
+
+
+def _value16(bits, dtype):
+    return from_bits16(bits, dtype).double().numpy()
+
+
+def _ulp_size16(bits, dtype):
+    """Spacing of the 16-bit format at each value (subnormal spacing below the normal range)."""
+    v = np.abs(_value16(bits, dtype))
+    mant, emin = (10, -14) if dtype == torch.float16 else (7, -126)
+    e = np.floor(np.log2(np.maximum(v, 2.0 ** emin)))
+    return 2.0 ** (e - mant)
+
+
+def check_gradient_end_to_end(got_soft, got_grad, want_soft, v, t, name, dtype):
+    """The chain forward -> backward against the oracle's chain.
+
+    1. backward is exact arithmetic on the stored softmax: the GPU gradient must equal the oracle's
+       backward applied to the GPU's own stored softmax, bit for bit;
+    2. hence the GPU gradient can differ from the oracle's end-to-end gradient only where the stored
+       softmax differs (<= 1 ulp, rare), and there by no more than that one softmax step times
+       |grad_output| plus the final rounding.  (An fp16 softmax of a 32,000-class row is mostly
+       subnormal, so one step of it can be several ulps of the scaled-up gradient.)"""
+    same_input = got_soft.copy()
+    oracle.ce_backward_inplace(v, t, same_input, -100, name)
+    assert np.array_equal(got_grad, same_input)
+    end_to_end = want_soft.copy()
+    oracle.ce_backward_inplace(v, t, end_to_end, -100, name)
+    differs = got_grad != end_to_end
+    assert not np.any(differs & (got_soft == want_soft))
+    assert differs.mean() < 1e-3
+    if differs.any():
+        err = np.abs(_value16(got_grad, dtype) - _value16(end_to_end, dtype))
+        bound = _ulp_size16(want_soft, dtype) * np.abs(v.astype(np.float64))[:, None] + _ulp_size16(end_to_end, dtype)
+        assert np.all(err[differs] <= bound[differs])
+    return differs.mean()
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+@pytest.mark.parametrize("n", [1000, 32000, 128256])
+def test_forward_backward_chain(name, dtype, n):
+    """Gradients through both kernels vs the oracle through both restatements, at the upstream scales
+    training uses (at 1.0 most fp16 gradients of a 16k-row mean are below the subnormal range)."""
+    m = 9
+    x, t = _case(m, n, dtype, seed=n + 2, ignore_frac=0.3)
+    valid = (t != -100).float()
+    want_soft, _ = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
+    for upstream in (1.0, 32768.0, 2.0 ** 20):
+        v = (valid / valid.sum() * upstream / 1024).float()      # mean over a 1024x larger batch
+        softmax, _ = _forward_gpu(x, t)
+        got_soft = bits16(softmax)
+        assert ulp_distance16(got_soft, want_soft).max() <= 1
+        F.cross_entropy_backward_inplace(m, n, v.cuda(), t.cuda(), softmax, -100)
+        got = bits16(softmax)
+        check_gradient_end_to_end(got_soft, got, want_soft, v.numpy(), t.numpy(), name, dtype)
+        assert np.all(got[t.numpy() == -100] == 0)
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_special_rows(name, dtype):
+    n = 64
+    rows = [
+        torch.full((n,), float("-inf")),                 # M clamps to -1e6, S = 1e-10
+        torch.full((n,), 0.5),                           # uniform
+        torch.cat([torch.tensor([60000.0 if dtype == torch.float16 else 3e38]), torch.zeros(n - 1)]),
+        torch.cat([torch.tensor([float("nan")]), torch.ones(n - 1)]),
+        torch.cat([torch.tensor([float("inf")]), torch.ones(n - 1)]),
+        torch.linspace(-30, 30, n),
+    ]
+    x = torch.stack(rows).to(dtype)
+    t = torch.tensor([0, 5, 0, 3, 0, n - 1], dtype=torch.int32)
+    softmax, loss = _forward_gpu(x, t)
+    want_soft, want_loss = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
+    got = from_bits16(bits16(softmax), dtype).float().numpy()
+    want = from_bits16(want_soft, dtype).float().numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert ulp_distance16(bits16(softmax)[~np.isnan(got)], want_soft[~np.isnan(want)]).max() <= 1
+    np.testing.assert_allclose(loss.cpu().numpy(), want_loss, rtol=2e-6, atol=1e-6, equal_nan=True)
+    # out-of-range target that is not ignore_index: NaN loss instead of an out-of-bounds read
+    _, loss = _forward_gpu(x[:2], torch.tensor([n, -7], dtype=torch.int32))
+    assert torch.isnan(loss).all()
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_unaligned_row_base_takes_the_element_kernel(name, dtype):
+    m, n = 6, 1024
+    x, t = _case(m, n, dtype, seed=3)
+    buf = torch.zeros(m * n + 8, dtype=dtype, device="cuda")
+    for off in (1, 4):
+        xg = buf[off:off + m * n].view(m, n)
+        xg.copy_(x)
+        soft_buf = torch.zeros(m * n + 8, dtype=dtype, device="cuda")
+        soft = soft_buf[off:off + m * n].view(m, n)
+        out = torch.empty(m, dtype=torch.float32, device="cuda")
+        F.cross_entropy_forward(m, n, xg, t.cuda(), soft, out, -100)
+        want_soft, want_loss = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
+        assert ulp_distance16(bits16(soft), want_soft).max() <= 1
+        assert soft_buf[:off].count_nonzero() == 0 and soft_buf[off + m * n:].count_nonzero() == 0
+        v = torch.rand(m)
+        want = bits16(soft)
+        oracle.ce_backward_inplace(v.numpy(), t.numpy(), want, -100, name)
+        F.cross_entropy_backward_inplace(m, n, v.cuda(), t.cuda(), soft, -100)
+        assert np.array_equal(bits16(soft), want)
+        assert soft_buf[:off].count_nonzero() == 0 and soft_buf[off + m * n:].count_nonzero() == 0
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_sumexp_and_softmax_inplace(name, dtype):
+    for m, n in ((5, 1000), (3, 32000), (4, 777)):
+        x, _ = _case(m, n, dtype, seed=n)
+        xg = x.cuda()
+        mx = xg.float().max(-1).values.contiguous()
+        se = F.fused_sumexp(xg, mx)
+        want_se = oracle.fused_sumexp(bits16(x), mx.cpu().numpy(), name)
+        np.testing.assert_allclose(se.cpu().numpy(), want_se, rtol=2e-6)
+        want = bits16(x)
+        oracle.fused_softmax_inplace(want, mx.cpu().numpy(), want_se, name)
+        F.fused_softmax_inplace(xg, mx, torch.from_numpy(want_se).cuda())
+        assert ulp_distance16(bits16(xg), want).max() <= 1
+
+
+# ---- module level, shaped like the reference's tests/test_loss_func.py -----------------------
+def _run(x, tgt, loss_func, scale=32768, use_float=False):
+    x = x.clone().detach()
+    if use_float:
+        x = x.float()
+    x = x.requires_grad_()
+    loss = loss_func(x, tgt)
+    (loss * scale).backward()
+    return loss, x.grad
+
+
+def _check(x, tgt, fused, plain):
+    loss_1, grad_1 = _run(x, tgt, fused)
+    loss_2, grad_2 = _run(x, tgt, plain, use_float=True)
+    assert grad_1.isnan().sum() == 0 and grad_2.isnan().sum() == 0
+    assert (loss_1 - loss_2).abs().item() < 1e-5          # tests/test_loss_func.py:31
+    assert (grad_1 - grad_2).abs().max().item() < 1e-1    # tests/test_loss_func.py:32
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_module_against_torch_cross_entropy(dtype):
+    torch.manual_seed(0)
+    N = 32 * 512
+    for C in [10, 50, 90, 100, 500, 900, 1000, 5000, 16000, 30000]:
+        x = torch.randn(N, C).cuda().to(dtype)
+        tgt = torch.randint(0, C, (N,)).cuda().long()
+        _check(x, tgt, FusedCrossEntropy(), torch.nn.CrossEntropyLoss())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_module_with_class_weights_and_ignored_targets(dtype):
+    torch.manual_seed(1)
+    N = 32 * 512
+    for C in (10, 50, 100):
+        weight = (torch.randperm(C) + 1).cuda()
+        x = torch.randn(N, C).cuda().to(dtype)
+        tgt = torch.randint(0, C, (N,)).cuda().long()
+        tgt[torch.randint(0, 2, (N,)).cuda().bool()] = -100
+        _check(x, tgt, FusedCrossEntropy(weight=weight.clone().to(dtype)),
+               torch.nn.CrossEntropyLoss(weight=weight.clone().float()))
+        for reduction in ("none", "sum"):
+            a = FusedCrossEntropy(reduction=reduction)(x, tgt)
+            b = torch.nn.functional.cross_entropy(x.float(), tgt, reduction=reduction)
+            torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-4 if reduction == "none" else 1.0)
+
+
+def test_module_contract():
+    x = torch.randn(8, 16, device="cuda")
+    tgt = torch.randint(0, 16, (8,), device="cuda")
+    # fp32 input is torch's own cross entropy, label smoothing included
+    a = FusedCrossEntropy(label_smoothing=0.1)(x, tgt)
+    b = torch.nn.functional.cross_entropy(x, tgt, label_smoothing=0.1)
+    assert torch.equal(a, b)
+    with pytest.raises(ValueError):
+        FusedCrossEntropy(weight=torch.ones(3, device="cuda"))(x.half(), tgt)
+    with pytest.raises(AssertionError):
+        OpFusedCrossEntropy.apply(x.half()[0], tgt.int(), -100)
+    with pytest.raises(NotImplementedError):
+        FusedCrossEntropy(parallel=True)(x.half(), tgt)
+    # backward hands back the softmax buffer itself as the gradient
+    xh = x.half().requires_grad_()
+    out = OpFusedCrossEntropy.apply(xh, tgt.int(), -100)
+    out.sum().backward()
+    assert xh.grad.dtype == torch.float16 and xh.grad.shape == xh.shape
+    # all targets ignored: 0 / 0
+    assert torch.isnan(FusedCrossEntropy()(x.half(), torch.full((8,), -100, device="cuda")))
+
+
+def test_language_model_head_shape():
+    """16,384 rows x 32,000 classes fp16, 10 % ignored, mean reduction.  Seeded rows are checked
+    against the oracle; all rows are checked through row sums, the loss against torch in fp32 on
+    the GPU, and sign / zero structure of the gradient."""
+    m, n = 16384, 32000
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    x = (torch.randn(m, n, generator=gen, device="cuda") * 2).half()
+    t = torch.randint(0, n, (m,), generator=gen, device="cuda", dtype=torch.int32)
+    ignored = torch.randperm(m, generator=gen, device="cuda")[: m // 10]
+    t[ignored] = -100
+    softmax = torch.empty_like(x)
+    out = torch.empty(m, dtype=torch.float32, device="cuda")
+    F.cross_entropy_forward(m, n, x, t, softmax, out, -100)
+    rows = [0, 1, m - 1] + [int(r) for r in np.random.default_rng(3).integers(0, m, 13)]
+    idx = torch.tensor(rows, device="cuda")
+    want_soft, want_loss = oracle.ce_forward(bits16(x[idx]), t[idx].cpu().numpy(), -100, "fp16")
+    assert ulp_distance16(bits16(softmax[idx]), want_soft).max() <= 1
+    np.testing.assert_allclose(out[idx].cpu().numpy(), want_loss, rtol=2e-6, atol=2e-6)
+    sums = torch.zeros(m, device="cuda")
+    ref = torch.zeros(m, device="cuda")
+    for lo in range(0, m, 2048):
+        sums[lo:lo + 2048] = softmax[lo:lo + 2048].float().sum(-1)
+        ref[lo:lo + 2048] = torch.nn.functional.cross_entropy(x[lo:lo + 2048].float(), t[lo:lo + 2048].long(),
+                                                              ignore_index=-100, reduction="none")
+    assert (sums - 1).abs().max().item() < 2e-2            # fp16 rounding of 32,000 tiny terms
+    torch.testing.assert_close(out, ref, rtol=1e-3, atol=1e-5)
+    valid = (t != -100)
+    scale = 2.0 ** 20
+    v = (valid.float() / valid.sum() * scale)
+    got_soft = bits16(softmax[idx])
+    F.cross_entropy_backward_inplace(m, n, v, t, softmax, -100)
+    assert softmax[~valid].count_nonzero() == 0
+    check_gradient_end_to_end(got_soft, bits16(softmax[idx]), want_soft, v[idx].cpu().numpy(), t[idx].cpu().numpy(),
+                              "fp16", torch.float16)
+    tv = t[valid].long()
+    at_target = softmax[valid].gather(1, tv[:, None])
+    assert (at_target < 0).all()
+    del x, softmax
+    torch.cuda.empty_cache()

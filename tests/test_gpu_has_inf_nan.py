@@ -1,0 +1,142 @@
+"""has_inf_nan on the GPU, through the C ABI, against the oracle: bit-exact 0/1."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from bmtrain_amd.loss import _function as F
+from bmtrain_amd import C
+from conftest import bits16, from_bits16
+
+pytestmark = pytest.mark.gpu
+DTYPES = [("fp16", torch.float16), ("bf16", torch.bfloat16)]
+
+
+def gpu_flag(x, start=0):
+    out = torch.full((1,), start, dtype=torch.uint8, device="cuda")[0]
+    F.has_inf_nan(x, out)
+    return int(out.item())
+
+
+def oracle_flag(x, name, start=0):
+    out = np.array([start], np.uint8)
+    oracle.has_inf_nan(bits16(x), out, name)
+    return int(out[0])
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_every_bit_pattern(name, dtype):
+    """One launch per pattern, each on a one-element tensor, each with its own flag byte."""
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    x = from_bits16(bits, dtype).cuda()
+    flags = torch.zeros(65536, dtype=torch.uint8, device="cuda")
+    launcher = C.has_nan_inf_fp16_launcher if name == "fp16" else C.has_nan_inf_bf16_launcher
+    stream = torch.cuda.current_stream().cuda_stream
+    for i in range(65536):
+        launcher(1, x.data_ptr() + 2 * i, 0, flags.data_ptr() + i, stream)
+    got = flags.cpu().numpy()
+    want = np.zeros(65536, np.uint8)
+    for i in range(65536):
+        oracle.has_inf_nan(bits[i:i + 1], want[i:i + 1], name)
+    assert np.array_equal(got, want)
+    # and all the finite patterns together raise nothing
+    finite = from_bits16(bits[want == 0], dtype).cuda()
+    assert gpu_flag(finite) == 0
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_reference_style_sweep(name, dtype):
+    rnd = random.Random(1)
+    torch.manual_seed(1)
+    for n in list(range(1, 100)) + [1000] * 3 + [10000] * 3 + [100000] * 3 + [1000000] * 3:
+        x = torch.rand(n).to(dtype).cuda()
+        assert gpu_flag(x) == 0 == oracle_flag(x, name)
+        p = rnd.randint(0, n - 1)
+        x[p] = float("inf")
+        assert gpu_flag(x) == 1 == oracle_flag(x, name)
+        x[p] = 2
+        assert gpu_flag(x) == 0
+        x[rnd.randint(0, n - 1)] = float("nan")
+        assert gpu_flag(x) == 1
+        x[rnd.randint(0, n - 1)] = float("-inf")
+        x[rnd.randint(0, n - 1)] = float("inf")
+        assert gpu_flag(x) == 1 == oracle_flag(x, name)
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_unaligned_views_see_exactly_their_elements(name, dtype):
+    """A hit just outside the view must not count; a hit on its first or last element must."""
+    base = torch.ones(4096 + 64, dtype=dtype, device="cuda")
+    for off in range(0, 17):
+        for n in (1, 2, 7, 8, 9, 15, 16, 17, 255, 1024, 4000):
+            view = base[off:off + n]
+            base.fill_(1)
+            if off > 0:
+                base[off - 1] = float("inf")
+            base[off + n] = float("nan")
+            assert gpu_flag(view) == 0, (off, n)
+            base[off] = float("inf")
+            assert gpu_flag(view) == 1, (off, n)
+            base[off] = 1
+            base[off + n - 1] = float("nan")
+            assert gpu_flag(view) == 1, (off, n)
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_sticky_flag_and_empty_input(name, dtype):
+    x = torch.ones(1000, dtype=dtype, device="cuda")
+    assert gpu_flag(x, start=1) == 1           # never cleared
+    assert gpu_flag(x[:0], start=0) == 0       # n == 0 is a no-op
+    flag = torch.zeros(1, dtype=torch.uint8, device="cuda")[0]
+    bad = x.clone(); bad[123] = float("nan")
+    for t in (x, bad, x, x):                   # accumulated over tensors, as check_overflow does
+        F.has_inf_nan(t, flag)
+    assert flag.item() == 1
+
+
+def test_dtype_and_layout_errors():
+    out = torch.zeros(1, dtype=torch.uint8, device="cuda")[0]
+    with pytest.raises(ValueError):
+        F.has_inf_nan(torch.ones(4, device="cuda"), out)
+    with pytest.raises(AssertionError):
+        F.has_inf_nan(torch.ones(4, dtype=torch.float16), out)
+    with pytest.raises(AssertionError):
+        F.has_inf_nan(torch.ones(8, dtype=torch.float16, device="cuda")[::2], out)
+    with pytest.raises(AssertionError):
+        F.has_inf_nan(torch.ones(4, dtype=torch.float16, device="cuda"), torch.zeros(1, device="cuda"))
+
+
+def _fill_normal_(x, std, seed, chunk=1 << 28):
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    for lo in range(0, x.numel(), chunk):
+        part = x[lo:lo + chunk]
+        part.copy_(torch.randn(part.numel(), generator=gen, device="cuda", dtype=torch.float32).mul_(std))
+
+
+@pytest.mark.parametrize("name,dtype,n", [("bf16", torch.bfloat16, 6_738_415_616), ("fp16", torch.float16, 1 << 30)])
+def test_full_size_buffers(name, dtype, n):
+    """The gradient-buffer sizes of a 7B-parameter model: all finite -> 0; one +inf and one NaN
+    at seeded offsets (beyond 2^32 bytes for bf16) -> 1; each alone -> 1."""
+    x = torch.empty(n, dtype=dtype, device="cuda")
+    _fill_normal_(x, 1e-3, seed=2)
+    assert gpu_flag(x) == 0
+    rnd = random.Random(2)
+    a, b = rnd.randrange(n), rnd.randrange(n)
+    keep_a, keep_b = x[a].clone(), x[b].clone()
+    x[a] = float("inf")
+    assert gpu_flag(x) == 1
+    x[b] = float("nan")
+    assert gpu_flag(x) == 1
+    x[a] = keep_a
+    assert gpu_flag(x) == 1
+    x[b] = keep_b
+    assert gpu_flag(x) == 0
+    x[n - 1] = float("-inf")                    # very last element
+    assert gpu_flag(x) == 1
+    # a strided sample agrees with the oracle
+    sample = x[:: max(1, n // (1 << 20))].contiguous()
+    assert gpu_flag(sample) == oracle_flag(sample, name)
+    del x
+    torch.cuda.empty_cache()

@@ -1,0 +1,207 @@
+"""Optimizer classes and the loss-scale manager on the GPU, shaped like the reference's
+tests/test_optim.py and the overflow handling of bmtrain/optim/optim_manager.py."""
+import copy
+
+import pytest
+import torch
+
+import bmtrain_amd as bmt
+
+pytestmark = pytest.mark.gpu
+
+
+class TestModule(torch.nn.Module):
+    __test__ = False
+
+    def __init__(self):
+        super().__init__()
+        self.fc1 = torch.nn.Linear(128, 128, bias=False)
+        self.fc2 = torch.nn.Linear(128, 128)
+        self.fc3 = torch.nn.Linear(128, 128)
+        self.fc4 = torch.nn.Linear(128, 128)
+        self.fc5 = torch.nn.Linear(128, 128)
+        self.param = torch.nn.Parameter(torch.empty(1237))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_five_way_agreement(dtype):
+    """tests/test_optim.py:24-85: fused (16-bit), offload (16-bit), torch Adam (fp32), fused (fp32),
+    offload (fp32) on identical gradients, lr = 1, loss scale 4, 100 steps."""
+    torch.manual_seed(0)
+    models = [TestModule() for _ in range(5)]
+    state = models[0].state_dict()
+    for k in state:
+        state[k] = torch.randn_like(state[k])
+    for mdl in models:
+        mdl.load_state_dict(state)
+    model1, model2 = models[0].cuda().to(dtype), models[1].cuda().to(dtype)
+    model3, model4, model5 = (mdl.cuda() for mdl in models[2:])
+    opt1 = bmt.optim.AdamOptimizer(model1.parameters(), lr=1)
+    opt2 = bmt.optim.AdamOffloadOptimizer(model2.parameters(), lr=1)
+    opt3 = torch.optim.Adam(model3.parameters(), lr=1)
+    opt4 = bmt.optim.AdamOptimizer(model4.parameters(), lr=1)
+    opt5 = bmt.optim.AdamOffloadOptimizer(model5.parameters(), lr=1)
+    manager = bmt.optim.OptimManager(loss_scale=4)
+    for opt in (opt1, opt2, opt3, opt4, opt5):
+        manager.add_optimizer(opt)
+    for _ in range(100):
+        manager.zero_grad()
+        for p1, p2, p3, p4, p5 in zip(*(mdl.parameters() for mdl in (model1, model2, model3, model4, model5))):
+            grad = torch.randn_like(p1)
+            p1.grad = grad.to(dtype)
+            p2.grad = grad.to(dtype)
+            p3.grad = grad.float()
+            p4.grad = grad.float()
+            p5.grad = grad.float()
+        manager.step()
+        torch.cuda.synchronize()
+        for p1, p2, p3, p4, p5 in zip(*(mdl.parameters() for mdl in (model1, model2, model3, model4, model5))):
+            assert torch.abs(p1 - p2).max().item() < 1
+            assert torch.abs(p1 - p3).max().item() < 1
+            assert torch.abs(p2 - p3).max().item() < 1
+            assert torch.abs(p3 - p4).max().item() == 0
+            assert torch.abs(p3 - p5).max().item() < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_and_offload_agree_closely(dtype):
+    """Same expression on both sides (bf16: identical fp32 state, copy differs by rounding mode)."""
+    torch.manual_seed(1)
+    a = torch.nn.Parameter((torch.randn(10007) * 0.02).cuda().to(dtype))
+    b = torch.nn.Parameter(a.detach().clone())
+    opt_a = bmt.optim.AdamOptimizer([a], lr=1e-3, weight_decay=0.01)
+    opt_b = bmt.optim.AdamOffloadOptimizer([b], lr=1e-3, weight_decay=0.01, record_delta=True)
+    for _ in range(5):
+        g = (torch.randn(10007, device="cuda") * 1e-3 * 64).to(dtype)
+        a.grad = g.clone(); b.grad = g.clone()
+        opt_a.step(scale=64); opt_b.step(scale=64)
+        torch.cuda.synchronize()
+    pa = opt_a.state[a]["_param_fp32"].cpu()
+    pb = opt_b.state[b]["_param_fp32"]
+    if dtype == torch.bfloat16:
+        assert torch.equal(pa, pb)
+        assert torch.equal(opt_a.state[a]["exp_avg_sq"].cpu(), opt_b.state[b]["exp_avg_sq"])
+    else:   # the fused fp16 path keeps its first moment in fp16 (2^-11 relative rounding per step)
+        assert (pa - pb).abs().max() <= 1e-4 * pb.abs().max()
+    assert opt_b.get_avg_delta() != 0 and opt_b.get_var_delta() > 0
+    with pytest.raises(NotImplementedError):
+        bmt.optim.AdamOptimizer.get_avg_delta()
+
+
+def test_overflow_skips_the_step_and_halves_the_scale():
+    torch.manual_seed(2)
+    p = torch.nn.Parameter(torch.randn(1000, device="cuda").half())
+    opt = bmt.optim.AdamOptimizer([p], lr=1e-2)
+    manager = bmt.optim.OptimManager(loss_scale=1024, loss_scale_steps=2)
+    manager.add_optimizer(opt)
+    # a clean step creates state (moments stored multiplied by the scale)
+    p.grad = (torch.randn(1000, device="cuda") * 1024 * 1e-3).half()
+    manager.step()
+    before = p.detach().clone()
+    m_before = opt.state[p]["exp_avg"].clone()
+    v_before = opt.state[p]["exp_avg_sq"].clone()
+    assert opt.state[p]["step"] == 1
+    # overflow: skipped, scale halved, fp16 moments rescaled, grads zeroed
+    p.grad = (torch.randn(1000, device="cuda")).half()
+    p.grad[17] = float("inf")
+    manager.step()
+    assert manager.loss_scale == 512 and opt.state[p]["step"] == 1
+    assert torch.equal(p.detach(), before)
+    assert torch.equal(opt.state[p]["exp_avg"], m_before * 0.5)
+    assert torch.equal(opt.state[p]["exp_avg_sq"], v_before * 0.5)
+    assert p.grad.count_nonzero() == 0
+    # NaN too
+    p.grad[3] = float("nan")
+    manager.step()
+    assert manager.loss_scale == 256
+    # two clean steps grow it again
+    for _ in range(2):
+        p.grad = (torch.randn(1000, device="cuda") * 1e-3).half()
+        manager.step()
+    assert manager.loss_scale == 512 and opt.state[p]["step"] == 3
+    # never below min_loss_scale
+    manager2 = bmt.optim.OptimManager(loss_scale=1, min_loss_scale=1)
+    manager2.add_optimizer(opt)
+    p.grad = torch.full_like(p, float("nan"))
+    manager2.step()
+    assert manager2.loss_scale == 1
+    # fp32 parameters are not scanned (optim_manager.py:15)
+    q = torch.nn.Parameter(torch.randn(10, device="cuda"))
+    q.grad = torch.full_like(q, float("inf"))
+    bmt.optim.optim_manager.check_overflow([{"params": [q]}])
+    p.grad = torch.full_like(p, float("nan"))
+    with pytest.raises(OverflowError):
+        bmt.optim.optim_manager.check_overflow([{"params": [p]}])
+
+
+def test_hold_steps_and_maximize():
+    p = torch.nn.Parameter(torch.ones(64, device="cuda").bfloat16())
+    opt = bmt.optim.AdamOptimizer([p], lr=0.1, hold_steps=3)
+    for i in range(1, 5):
+        p.grad = torch.ones_like(p)
+        opt.step()
+        # lr is 0 while step < hold_steps, tested after the increment (adam.py:145,155)
+        assert (p.detach().float() == 1).all() == (i < 3)
+    q = torch.nn.Parameter(torch.zeros(64, device="cuda").bfloat16())
+    opt = bmt.optim.AdamOptimizer([{"params": [q], "maximize": True}], lr=0.1)
+    q.grad = torch.ones_like(q)
+    opt.step()
+    assert (q.detach() > 0).all()
+
+
+def test_state_dict_round_trip_resumes_exactly():
+    """tests/test_optim_state.py: a reloaded optimizer continues bit-identically."""
+    torch.manual_seed(4)
+    for cls in (bmt.optim.AdamOptimizer, bmt.optim.AdamOffloadOptimizer):
+        for dtype in (torch.float16, torch.bfloat16, torch.float32):
+            p = torch.nn.Parameter((torch.randn(513, device="cuda") * 0.1).to(dtype))
+            q = torch.nn.Parameter(p.detach().clone())
+            opt_p, opt_q = cls([p], lr=1e-2, weight_decay=0.1), cls([q], lr=1e-2, weight_decay=0.1)
+            mp, mq = bmt.optim.OptimManager(loss_scale=8), bmt.optim.OptimManager(loss_scale=2)
+            mp.add_optimizer(opt_p); mq.add_optimizer(opt_q)
+            grads = [(torch.randn(513, device="cuda") * 8).to(dtype) for _ in range(4)]
+            for g in grads[:2]:
+                p.grad = g.clone(); mp.step()
+            saved = copy.deepcopy(mp.state_dict())
+            assert set(saved["optimizers"][0]["state"][0]) >= {"step", "exp_avg", "exp_avg_sq"}
+            if dtype != torch.float32 or cls is bmt.optim.AdamOffloadOptimizer:
+                assert "_param_fp32" in saved["optimizers"][0]["state"][0]
+            q.data.copy_(p.data)
+            mq.load_state_dict(saved)
+            assert mq.loss_scale == 8
+            st = opt_q.state[q]
+            if cls is bmt.optim.AdamOptimizer:
+                assert st["exp_avg"].dtype == (torch.float16 if dtype == torch.float16 else torch.float32)
+                assert st["exp_avg_sq"].dtype == torch.float32 and st["exp_avg"].is_cuda
+            else:
+                assert not st["exp_avg"].is_cuda
+            for g in grads[2:]:
+                p.grad = g.clone(); q.grad = g.clone()
+                mp.step(); mq.step()
+            torch.cuda.synchronize()
+            assert torch.equal(p.detach(), q.detach()), (cls.__name__, dtype)
+
+
+def test_clip_grad_norm():
+    torch.manual_seed(5)
+    ps = [torch.nn.Parameter(torch.randn(100, device="cuda").half()) for _ in range(3)]
+    manager = bmt.optim.OptimManager(loss_scale=16)
+    for p in ps:
+        p.grad = (torch.randn(100, device="cuda") * 16).half()
+    want = torch.cat([p.grad.float() for p in ps]).norm() / 16
+    got = manager.clip_grad_norm([{"params": ps}], max_norm=1.0)
+    torch.testing.assert_close(got, want, rtol=1e-3, atol=1e-3)
+    after = torch.cat([p.grad.float() for p in ps]).norm() / 16
+    assert abs(after.item() - 1.0) < 1e-2
+
+
+def test_constructor_validation():
+    p = [torch.nn.Parameter(torch.zeros(1))]
+    for cls in (bmt.optim.AdamOptimizer, bmt.optim.AdamOffloadOptimizer):
+        for kw in (dict(lr=-1), dict(eps=-1), dict(betas=(1.0, 0.9)), dict(betas=(0.9, -0.1)), dict(weight_decay=-1)):
+            with pytest.raises(ValueError):
+                cls(p, **kw)
+    q = torch.nn.Parameter(torch.zeros(4, device="cuda", dtype=torch.float64))
+    q.grad = torch.zeros_like(q)
+    with pytest.raises(RuntimeError):
+        bmt.optim.AdamOptimizer([q]).step()
