@@ -209,8 +209,9 @@ __global__ __launch_bounds__(kSweepThreads) void ce_forward_sweep_kernel(
 
 // ---- element-wise kernels over the flat [m * n] array -----------------------------
 // OP 0: backward in place.  OP 1: softmax in place from given max / sum.
-constexpr int kFlatThreads = 256;
-constexpr int kFlatUnroll = 4;
+constexpr int kFlatThreads = 1024;
+constexpr int kFlatUnroll = 1;
+constexpr int kFlatScalarThreads = 256;
 
 template <typename T, int OP>
 __device__ __forceinline__ float flat_elem(float s, bool is_target, float a, float b) {
@@ -218,53 +219,51 @@ __device__ __forceinline__ float flat_elem(float s, bool is_target, float a, flo
     return expf(s - a) / b;                                 // a = max, b = sum
 }
 
+// One workgroup transforms one tile of kFlatThreads * kFlatUnroll vectors and exits.
 template <typename T, int OP>
 __global__ __launch_bounds__(kFlatThreads) void ce_flat_vec_kernel(
     int32_t nvec, int64_t total_vec, uint16_t *__restrict__ x, const float *__restrict__ row_a,
     const float *__restrict__ row_b, const int32_t *__restrict__ target) {
     u32x4 *xv = (u32x4 *)x;
-    const int64_t tile = (int64_t)kFlatThreads * kFlatUnroll;
-    const int64_t ntiles = (total_vec + tile - 1) / tile;
-    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-        const int64_t start = t * tile;
-        const int64_t row0 = start / nvec;
-        const uint32_t col0 = (uint32_t)(start - row0 * nvec);
-        u32x4 w[kFlatUnroll];
-        bool ok[kFlatUnroll];
+    const int64_t start = (int64_t)blockIdx.x * (kFlatThreads * kFlatUnroll);
+    const int64_t row0 = start / nvec;
+    const uint32_t col0 = (uint32_t)(start - row0 * nvec);
+    u32x4 w[kFlatUnroll];
+    bool ok[kFlatUnroll];
 #pragma unroll
-        for (int u = 0; u < kFlatUnroll; u++) {
-            const int64_t g = start + (int64_t)u * kFlatThreads + threadIdx.x;
-            ok[u] = g < total_vec;
-            if (ok[u]) w[u] = __builtin_nontemporal_load(xv + g);
+    for (int u = 0; u < kFlatUnroll; u++) {
+        const int64_t g = start + (int64_t)u * kFlatThreads + threadIdx.x;
+        ok[u] = g < total_vec;
+        if (ok[u]) w[u] = __builtin_nontemporal_load(xv + g);
+    }
+#pragma unroll
+    for (int u = 0; u < kFlatUnroll; u++) {
+        if (!ok[u]) continue;
+        const int64_t g = start + (int64_t)u * kFlatThreads + threadIdx.x;
+        const uint32_t off = col0 + (uint32_t)(u * kFlatThreads + threadIdx.x);
+        const uint32_t dr = off / (uint32_t)nvec;
+        const int64_t row = row0 + dr;
+        const int32_t col = (int32_t)(off - dr * (uint32_t)nvec) * 8;
+        const float a = row_a[row];
+        const float b = OP == 1 ? row_b[row] : 0.f;
+        const int32_t tk = OP == 0 ? target[row] - col : -1;  // position of the target inside this vector
+        u32x4 o;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const float lo = flat_elem<T, OP>(lo_f32<T>(w[u][k]), tk == 2 * k, a, b);
+            const float hi = flat_elem<T, OP>(hi_f32<T>(w[u][k]), tk == 2 * k + 1, a, b);
+            o[k] = pack2<T>(lo, hi);
         }
-#pragma unroll
-        for (int u = 0; u < kFlatUnroll; u++) {
-            if (!ok[u]) continue;
-            const int64_t g = start + (int64_t)u * kFlatThreads + threadIdx.x;
-            const uint32_t off = col0 + (uint32_t)(u * kFlatThreads + threadIdx.x);
-            const uint32_t dr = off / (uint32_t)nvec;
-            const int64_t row = row0 + dr;
-            const int32_t col = (int32_t)(off - dr * (uint32_t)nvec) * 8;
-            const float a = row_a[row];
-            const float b = OP == 1 ? row_b[row] : 0.f;
-            const int32_t tk = OP == 0 ? target[row] - col : -1;  // position of the target inside this vector
-            u32x4 o;
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const float lo = flat_elem<T, OP>(lo_f32<T>(w[u][k]), tk == 2 * k, a, b);
-                const float hi = flat_elem<T, OP>(hi_f32<T>(w[u][k]), tk == 2 * k + 1, a, b);
-                o[k] = pack2<T>(lo, hi);
-            }
-            __builtin_nontemporal_store(o, xv + g);
-        }
+        __builtin_nontemporal_store(o, xv + g);
     }
 }
 
 template <typename T, int OP>
-__global__ __launch_bounds__(kFlatThreads) void ce_flat_scalar_kernel(
+__global__ __launch_bounds__(kFlatScalarThreads) void ce_flat_scalar_kernel(
     int32_t n, int64_t total, uint16_t *__restrict__ x, const float *__restrict__ row_a,
     const float *__restrict__ row_b, const int32_t *__restrict__ target) {
-    for (int64_t g = (int64_t)blockIdx.x * kFlatThreads + threadIdx.x; g < total; g += (int64_t)gridDim.x * kFlatThreads) {
+    for (int64_t g = (int64_t)blockIdx.x * kFlatScalarThreads + threadIdx.x; g < total;
+         g += (int64_t)gridDim.x * kFlatScalarThreads) {
         const int64_t row = g / n;
         const int32_t col = (int32_t)(g - row * n);
         const float a = row_a[row];
@@ -364,12 +363,13 @@ static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void 
     if (rows_vectorisable(n, x)) {
         const int32_t nvec = n / 8;
         const int64_t total = (int64_t)m * nvec;
-        hipLaunchKernelGGL((ce_flat_vec_kernel<T, OP>), dim3(flat_grid(total, kFlatThreads * kFlatUnroll)), dim3(kFlatThreads),
-                           0, s, nvec, total, (uint16_t *)x, (const float *)row_a, (const float *)row_b,
-                           (const int32_t *)target);
+        const int64_t tiles = (total + kFlatThreads * kFlatUnroll - 1) / (kFlatThreads * kFlatUnroll);
+        if (tiles > 0x7FFFFFFF) return fail(-1, "cross_entropy launcher: tensor too large for one launch");
+        hipLaunchKernelGGL((ce_flat_vec_kernel<T, OP>), dim3((unsigned)tiles), dim3(kFlatThreads), 0, s, nvec, total,
+                           (uint16_t *)x, (const float *)row_a, (const float *)row_b, (const int32_t *)target);
     } else {
         const int64_t total = (int64_t)m * n;
-        hipLaunchKernelGGL((ce_flat_scalar_kernel<T, OP>), dim3(flat_grid(total, kFlatThreads)), dim3(kFlatThreads), 0, s, n,
+        hipLaunchKernelGGL((ce_flat_scalar_kernel<T, OP>), dim3(flat_grid(total, kFlatScalarThreads)), dim3(kFlatScalarThreads), 0, s, n,
                            total, (uint16_t *)x, (const float *)row_a, (const float *)row_b, (const int32_t *)target);
     }
     hipError_t e = hipGetLastError();

@@ -17,7 +17,10 @@
 
 namespace bmt {
 
-constexpr int kScanThreads = 256;
+// One workgroup scans one tile of kScanThreads * UNROLL 16-byte vectors and exits (short
+// workgroups stream faster here than a resident grid that loops).
+constexpr int kScanThreads = 1024;
+constexpr int kScanUnroll = 2;
 
 template <typename T>
 __device__ __forceinline__ uint32_t exp_all_ones2(uint32_t w) {
@@ -29,29 +32,17 @@ __global__ __launch_bounds__(kScanThreads) void has_inf_nan_kernel(
     const uint16_t *__restrict__ g, int64_t head, int64_t nvec, int64_t n, uint8_t *__restrict__ out) {
     uint32_t hit = 0;
     const u32x4 *body = (const u32x4 *)(g + head);
-    const int64_t tile = (int64_t)kScanThreads * UNROLL;
-    const int64_t ntiles = (nvec + tile - 1) / tile;
-    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-        const int64_t base = t * tile + threadIdx.x;
-        if (t * tile + tile <= nvec) {
-            u32x4 w[UNROLL];
+    const int64_t base = (int64_t)blockIdx.x * (kScanThreads * UNROLL) + threadIdx.x;
+    u32x4 w[UNROLL];
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++) w[u] = __builtin_nontemporal_load(body + base + (int64_t)u * kScanThreads);
-#pragma unroll
-            for (int u = 0; u < UNROLL; u++)
-                hit |= exp_all_ones2<T>(w[u].x) | exp_all_ones2<T>(w[u].y) | exp_all_ones2<T>(w[u].z) |
-                       exp_all_ones2<T>(w[u].w);
-        } else {
-#pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                const int64_t i = base + (int64_t)u * kScanThreads;
-                if (i < nvec) {
-                    u32x4 w = __builtin_nontemporal_load(body + i);
-                    hit |= exp_all_ones2<T>(w.x) | exp_all_ones2<T>(w.y) | exp_all_ones2<T>(w.z) | exp_all_ones2<T>(w.w);
-                }
-            }
-        }
+    for (int u = 0; u < UNROLL; u++) {
+        const int64_t i = base + (int64_t)u * kScanThreads;
+        if (i < nvec) w[u] = __builtin_nontemporal_load(body + i);
+        else w[u] = u32x4{0u, 0u, 0u, 0u};
     }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++)
+        hit |= exp_all_ones2<T>(w[u].x) | exp_all_ones2<T>(w[u].y) | exp_all_ones2<T>(w[u].z) | exp_all_ones2<T>(w[u].w);
     // Unaligned head (< 8 elements) and tail (< 8 elements): workgroup 0, one element per lane.
     if (blockIdx.x == 0) {
         const int64_t tail_lo = head + nvec * 8;
@@ -80,12 +71,11 @@ static int scan(int64_t n, const void *g, void *out, void *stream, const char *w
     int64_t head = (int64_t)(((16 - (a & 15u)) & 15u) / 2);
     if (head > n) head = n;
     const int64_t nvec = (n - head) / 8;
-    constexpr int UNROLL = 4;
+    constexpr int UNROLL = kScanUnroll;
     const int64_t tile = (int64_t)kScanThreads * UNROLL;
     const int64_t ntiles = (nvec + tile - 1) / tile;
-    static const int per_cu = env_int("BMT_SCAN_BLOCKS_PER_CU", 8);
-    const int64_t cap = (int64_t)device_cu_count() * per_cu;
-    const int64_t grid = ntiles < 1 ? 1 : (ntiles < cap ? ntiles : cap);
+    if (ntiles > 0x7FFFFFFF) return fail(-1, "has_nan_inf launcher: buffer too large for one launch");
+    const int64_t grid = ntiles < 1 ? 1 : ntiles;
     hipLaunchKernelGGL((has_inf_nan_kernel<T, UNROLL>), dim3((unsigned)grid), dim3(kScanThreads), 0, (hipStream_t)stream,
                        (const uint16_t *)g, head, nvec, n, (uint8_t *)out);
     hipError_t e = hipGetLastError();
