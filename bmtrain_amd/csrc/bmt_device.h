@@ -52,9 +52,21 @@ __device__ __forceinline__ float lo_f32<BFloat16>(uint32_t packed) { return __bu
 template <>
 __device__ __forceinline__ float hi_f32<BFloat16>(uint32_t packed) { return __builtin_bit_cast(float, packed & 0xFFFF0000u); }
 
+// Two fp32 values -> one dword of two 16-bit values, round-to-nearest-even, with the packed
+// hardware converts of gfx950 (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32).
+typedef float  f32x2_t  __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 template <typename T>
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    return (uint32_t)T::from_f32(lo) | ((uint32_t)T::from_f32(hi) << 16);
+__device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <>
+__device__ __forceinline__ uint32_t pack2<BFloat16>(float lo, float hi) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<Half>(float lo, float hi) {
+    asm("" : "+v"(lo), "+v"(hi));   // keep the fp32 rounding step (see Half::from_f32)
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, f16x2_t));
 }
 
 // ---- wave64 reductions ----------------------------------------------------

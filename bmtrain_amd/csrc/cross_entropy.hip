@@ -29,6 +29,60 @@ template <> __device__ __forceinline__ uint32_t neg_inf2<BFloat16>() { return 0x
 
 __device__ __forceinline__ float add_tiny(float s) { return (float)((double)s + 1e-10); }  // cross_entropy.cu:28
 
+// ---- exponentials and the quotient -------------------------------------------------
+// All exponentials here are e^(x - M) with x <= M.  They are produced multiplied by 2^64
+// ("biased"): v_exp_f32 returns 0 for results below 2^-126, and the bias keeps everything that
+// can still matter after the division (down to 2^-190) in the normal range; the factor is
+// removed again, exactly, by the reciprocal used for the quotient.
+constexpr float kLog2e = 1.44269502162933349609375f;       // fp32 nearest to log2(e)
+constexpr float kLog2eLo = 1.925963033500011e-08f;          // log2(e) - kLog2e
+constexpr float kLn2 = 0.693147182464599609375f;
+constexpr float kBias = 64.0f;
+constexpr float kTwoPowBias = 18446744073709551616.0f;      // 2^64
+constexpr float kTwoPowMinusBias = 5.42101086242752217e-20f;  // 2^-64
+
+// 2^64 * e^(x - M), accurate to about 1.5 fp32 ulp: the product (x - M) * log2(e) is carried in
+// two floats (the rounding error of the product and the low part of log2(e)), and the low part
+// enters through e^lo ~ 1 + lo.  When x - M is -inf, or so negative that the product overflows,
+// the error term is NaN or inf while the result must be 0; v_med3_f32 maps both to a finite
+// value (with a NaN operand it returns the minimum of the others), and 0 * finite = 0.  A NaN
+// argument still yields NaN through v_exp_f32.
+__device__ __forceinline__ float exp_biased(float x, float M) {
+    const float d = x - M;
+    const float t = d * kLog2e;
+    float lo = __builtin_fmaf(d, kLog2e, -t);
+    lo = __builtin_fmaf(d, kLog2eLo, lo);
+    lo = __builtin_amdgcn_fmed3f(lo, -1.0f, 1.0f);
+    const float e = __builtin_amdgcn_exp2f(t + kBias);
+    return __builtin_fmaf(e, lo * kLn2, e);
+}
+// Same quantity from one fma and one v_exp_f32 (relative error up to about 2^-19); used only
+// where the values are summed.  `c` = 64 - M * log2(e).
+__device__ __forceinline__ float exp_biased_fast(float x, float c) {
+    return __builtin_amdgcn_exp2f(__builtin_fmaf(x, kLog2e, c));
+}
+
+// The row's divisor in the three forms the kernels need.
+struct RowSum {
+    float S;      // sum of exponentials + 1e-10, unbiased (for the loss)
+    float S64;    // S * 2^64: the divisor of the biased exponentials
+    float r64;    // correctly rounded 1 / S64
+};
+__device__ __forceinline__ RowSum make_row_sum(float biased_sum) {
+    RowSum rs;
+    rs.S = add_tiny(biased_sum * kTwoPowMinusBias);
+    rs.S64 = rs.S * kTwoPowBias;
+    rs.r64 = (1.0f / rs.S) * kTwoPowMinusBias;
+    return rs;
+}
+// e / S, correctly rounded, from the reciprocal: one Newton correction of the product with the
+// exact remainder (Markstein); equal to the IEEE quotient the reference computes.
+__device__ __forceinline__ float quotient(float e_biased, const RowSum &rs) {
+    const float q = e_biased * rs.r64;
+    const float rem = __builtin_fmaf(-q, rs.S64, e_biased);
+    return __builtin_fmaf(rem, rs.r64, q);
+}
+
 // Loss of one row; an out-of-range target that is not ignore_index yields NaN instead
 // of the reference's out-of-bounds read.
 template <typename T>
@@ -80,7 +134,7 @@ __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
     for (int c = 0; c < CHUNKS; c++) {
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            const float a = expf(lo_f32<T>(w[c][k]) - M), b = expf(hi_f32<T>(w[c][k]) - M);
+            const float a = exp_biased(lo_f32<T>(w[c][k]), M), b = exp_biased(hi_f32<T>(w[c][k]), M);
             sum += a; sum += b;
             if (KEEP_EXP) { e[c][2 * k] = a; e[c][2 * k + 1] = b; }
         }
@@ -88,7 +142,8 @@ __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
         // the temporaries of many chunks, which would spill the row.
         if (!KEEP_EXP) __builtin_amdgcn_sched_barrier(0);
     }
-    const float S = add_tiny(block_allreduce<false>(sum, slots[1]));
+    const RowSum rs = make_row_sum(block_allreduce<false>(sum, slots[1]));
+    const float S = rs.S;
 
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
@@ -97,9 +152,9 @@ __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
             u32x4 o;
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                const float a = KEEP_EXP ? e[c][2 * k] : expf(lo_f32<T>(w[c][k]) - M);
-                const float b = KEEP_EXP ? e[c][2 * k + 1] : expf(hi_f32<T>(w[c][k]) - M);
-                o[k] = pack2<T>(a / S, b / S);
+                const float a = KEEP_EXP ? e[c][2 * k] : exp_biased(lo_f32<T>(w[c][k]), M);
+                const float b = KEEP_EXP ? e[c][2 * k + 1] : exp_biased(hi_f32<T>(w[c][k]), M);
+                o[k] = pack2<T>(quotient(a, rs), quotient(b, rs));
             }
             __builtin_nontemporal_store(o, sr + j);
         }
@@ -119,15 +174,16 @@ __device__ __forceinline__ void vec_max(const u32x4 &w, float &mx) {
     for (int k = 0; k < 4; k++) { mx = fmaxf(lo_f32<T>(w[k]), mx); mx = fmaxf(hi_f32<T>(w[k]), mx); }
 }
 template <typename T>
-__device__ __forceinline__ void vec_sumexp(const u32x4 &w, float M, float &sum) {
+__device__ __forceinline__ void vec_sumexp(const u32x4 &w, float c, float &sum) {
 #pragma unroll
-    for (int k = 0; k < 4; k++) { sum += expf(lo_f32<T>(w[k]) - M); sum += expf(hi_f32<T>(w[k]) - M); }
+    for (int k = 0; k < 4; k++) { sum += exp_biased_fast(lo_f32<T>(w[k]), c); sum += exp_biased_fast(hi_f32<T>(w[k]), c); }
 }
 template <typename T>
-__device__ __forceinline__ u32x4 vec_softmax(const u32x4 &w, float M, float S) {
+__device__ __forceinline__ u32x4 vec_softmax(const u32x4 &w, float M, const RowSum &rs) {
     u32x4 o;
 #pragma unroll
-    for (int k = 0; k < 4; k++) o[k] = pack2<T>(expf(lo_f32<T>(w[k]) - M) / S, expf(hi_f32<T>(w[k]) - M) / S);
+    for (int k = 0; k < 4; k++)
+        o[k] = pack2<T>(quotient(exp_biased(lo_f32<T>(w[k]), M), rs), quotient(exp_biased(hi_f32<T>(w[k]), M), rs));
     return o;
 }
 
@@ -165,22 +221,24 @@ __global__ __launch_bounds__(kLongThreads) void ce_forward_long_kernel(
     const float M = fmaxf(block_allreduce<true>(mx, slots[0]), -1e6f);
 
     float sum = 0.f;
+    const float cexp = __builtin_fmaf(-M, kLog2e, kBias);
 #pragma unroll
-    for (int c = 0; c < REG; c++) { vec_sumexp<T>(w[c], M, sum); __builtin_amdgcn_sched_barrier(0); }
+    for (int c = 0; c < REG; c++) { vec_sumexp<T>(w[c], cexp, sum); __builtin_amdgcn_sched_barrier(0); }
 #pragma unroll 1
-    for (int c = 0; c < LDSC; c++) vec_sumexp<T>(staged[c * kLongThreads + tid], M, sum);
-    const float S = add_tiny(block_allreduce<false>(sum, slots[1]));
+    for (int c = 0; c < LDSC; c++) vec_sumexp<T>(staged[c * kLongThreads + tid], cexp, sum);
+    const RowSum rs = make_row_sum(block_allreduce<false>(sum, slots[1]));
+    const float S = rs.S;
 
 #pragma unroll
     for (int c = 0; c < REG; c++) {
         const int j = c * kLongThreads + tid;
-        if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(w[c], M, S), sr + j);
+        if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(w[c], M, rs), sr + j);
         __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll 1
     for (int c = 0; c < LDSC; c++) {
         const int j = (REG + c) * kLongThreads + tid;
-        if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(staged[c * kLongThreads + tid], M, S), sr + j);
+        if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(staged[c * kLongThreads + tid], M, rs), sr + j);
     }
     if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, S);
 }
@@ -201,9 +259,10 @@ __global__ __launch_bounds__(kSweepThreads) void ce_forward_sweep_kernel(
     for (int i = threadIdx.x; i < n; i += kSweepThreads) mx = fmaxf(T::to_f32(xr[i]), mx);
     const float M = fmaxf(block_allreduce<true>(mx, slots[0]), -1e6f);
     float sum = 0.f;
-    for (int i = threadIdx.x; i < n; i += kSweepThreads) sum += expf(T::to_f32(xr[i]) - M);
-    const float S = add_tiny(block_allreduce<false>(sum, slots[1]));
-    for (int i = threadIdx.x; i < n; i += kSweepThreads) sr[i] = T::from_f32(expf(T::to_f32(xr[i]) - M) / S);
+    for (int i = threadIdx.x; i < n; i += kSweepThreads) sum += exp_biased(T::to_f32(xr[i]), M);
+    const RowSum rs = make_row_sum(block_allreduce<false>(sum, slots[1]));
+    const float S = rs.S;
+    for (int i = threadIdx.x; i < n; i += kSweepThreads) sr[i] = T::from_f32(quotient(exp_biased(T::to_f32(xr[i]), M), rs));
     if (threadIdx.x == 0) out[row] = row_loss<T>(xr, n, target[row], ignore_index, M, S);
 }
 
