@@ -1,5 +1,4 @@
-// Host-side helpers shared by the launchers: per-thread error text, device
-// properties, environment overrides used when tuning launch shapes.
+// Host-side helpers shared by the launchers: per-thread error text, device properties.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -14,8 +13,5 @@ int fail_message(int code, const char *what);
 
 // Number of compute units of the current device (cached per device).
 int device_cu_count();
-
-// Integer from the environment, or `fallback` when unset / malformed.
-int env_int(const char *name, int fallback);
 
 }  // namespace bmt

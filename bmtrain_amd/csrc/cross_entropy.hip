@@ -6,14 +6,17 @@
 //   M = max(max_i x_i, -1e6);  S = sum_i expf(x_i - M) + 1e-10
 //   softmax[r, i] = to16(expf(x_i - M) / S)
 //   out[r] = target[r] != ignore ? (-x[target[r]] + M) + logf(S) : 0
-// The reference walks each row three times from global memory.  Here a row is read
-// from HBM once, as 16-byte vectors, into the registers of the workgroup that owns
-// it; the maximum, the exponentials (kept in fp32 registers when they fit, else
-// recomputed from the packed row), the sum and the quotient all work on registers,
-// and the softmax goes out as 16-byte vectors.  Reductions are a wave64 butterfly
-// followed by one LDS slot per wave.  Rows whose length is not a multiple of 8 or
-// whose base is not 16-byte aligned, and rows too long for the register file, take a
-// three-sweep kernel with element loads that relies on L2 for the re-reads.
+// The reference walks each row three times from global memory.  Here one workgroup owns a
+// row and moves it as 16-byte vectors:
+//   * up to 32,768 elements the row is read once into registers; maximum, exponentials (kept in
+//     fp32 registers), sum and quotient all work on registers (ce_forward_row_kernel);
+//   * up to 131,072 elements the row is streamed once while a per-lane running maximum / sum is
+//     kept; 4 vectors per lane stay in registers and up to 4 in LDS, the remainder is fetched a
+//     second time for the output sweep (ce_forward_retain_kernel);
+//   * longer rows are streamed twice (ce_forward_stream_kernel).
+// Reductions are a wave64 butterfly followed by one LDS slot per wave.  Rows whose length is not
+// a multiple of 8 or whose base is not 16-byte aligned take a three-sweep kernel with element
+// loads (ce_forward_sweep_kernel).
 //
 // Backward (reference kernels :46-60, :104-121), element-wise and in place on the
 // stored softmax: x[r, i] = to16((x[r, i] - (i == target[r])) * grad_output[r]).
@@ -163,11 +166,14 @@ __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
     if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, S);
 }
 
-// ---- forward, long rows: registers + LDS ---------------------------------------
-// A row of up to (REG + LDSC) * 8192 elements is held on chip by one 1024-lane
-// workgroup: REG vectors per lane stay in registers, LDSC more per lane sit in LDS
-// (lane-contiguous 16-byte slots, conflict-free).  Used when the row does not fit
-// the register file alone; exponentials are recomputed in the output sweep.
+// ---- helpers on one 16-byte vector (8 elements) ------------------------------------------
+// Returns `w` through an empty asm: the compiler then cannot keep the unpacked fp32 values of
+// one sweep alive for the next one, which would double the registers a resident row occupies.
+__device__ __forceinline__ u32x4 reread(u32x4 w) {
+    asm volatile("" : "+v"(w));
+    return w;
+}
+
 template <typename T>
 __device__ __forceinline__ void vec_max(const u32x4 &w, float &mx) {
 #pragma unroll
@@ -187,13 +193,17 @@ __device__ __forceinline__ u32x4 vec_softmax(const u32x4 &w, float M, const RowS
     return o;
 }
 
-constexpr int kLongThreads = 1024;
-template <typename T, int REG, int LDSC>
-__global__ __launch_bounds__(kLongThreads) void ce_forward_long_kernel(
+// ---- forward, long rows: two sweeps, the second one served by the caches ------------
+// Sweep 1 reads the row from HBM and keeps, per lane, a running maximum and the sum of
+// exponentials relative to it (rescaled when the maximum grows); nothing is stored on chip,
+// so several workgroups per CU overlap their memory and ALU phases.  Sweep 2 reads the row
+// again — it was just fetched with the default cache policy, so L2 / Infinity Cache still hold
+// it — and writes the quotient.  THREADS lanes per row, UNROLL vectors per lane per step.
+template <typename T, int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void ce_forward_stream_kernel(
     int32_t n, int32_t nvec, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
     uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
-    extern __shared__ u32x4 staged[];  // LDSC * 1024 vectors
-    __shared__ float slots[2][kLongThreads / kWave];
+    __shared__ float slots[2][THREADS / kWave];
     const int64_t row = blockIdx.x;
     const u32x4 *xr = (const u32x4 *)(x + row * n);
     u32x4 *sr = (u32x4 *)(softmax + row * n);
@@ -201,46 +211,161 @@ __global__ __launch_bounds__(kLongThreads) void ce_forward_long_kernel(
     const uint32_t pad = neg_inf2<T>();
     const u32x4 pad4 = {pad, pad, pad, pad};
 
-    u32x4 w[REG];
+    float m = -1e6f;          // running maximum of this lane, never below the reference's clamp
+    float s = 0.f;            // sum of 2^64 * e^(x - m) over this lane's elements so far
+    float cexp = __builtin_fmaf(-m, kLog2e, kBias);
+    for (int j0 = 0; j0 < nvec; j0 += THREADS * UNROLL) {
+        u32x4 w[UNROLL];
 #pragma unroll
-    for (int c = 0; c < REG; c++) {
-        const int j = c * kLongThreads + tid;
-        w[c] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
+        for (int u = 0; u < UNROLL; u++) {
+            const int j = j0 + u * THREADS + tid;
+            w[u] = j < nvec ? xr[j] : pad4;
+        }
+        float vm = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) vec_max<T>(w[u], vm);
+        if (vm > m) {   // rare after the first steps
+            s *= __builtin_amdgcn_exp2f((m - vm) * kLog2e);
+            m = vm;
+            cexp = __builtin_fmaf(-m, kLog2e, kBias);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) vec_sumexp<T>(w[u], cexp, s);
     }
+    const float M = block_allreduce<true>(m, slots[0]);
+    s *= __builtin_amdgcn_exp2f((m - M) * kLog2e);
+    const RowSum rs = make_row_sum(block_allreduce<false>(s, slots[1]));
+
+    for (int j0 = 0; j0 < nvec; j0 += THREADS * UNROLL) {
+        u32x4 w[UNROLL];
 #pragma unroll
-    for (int c = 0; c < LDSC; c++) {
-        const int j = (REG + c) * kLongThreads + tid;
-        staged[c * kLongThreads + tid] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
+        for (int u = 0; u < UNROLL; u++) {
+            const int j = j0 + u * THREADS + tid;
+            w[u] = j < nvec ? xr[j] : pad4;
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const int j = j0 + u * THREADS + tid;
+            if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(w[u], M, rs), sr + j);
+        }
     }
-    // Every lane reads back only the LDS slots it wrote itself: no barrier is needed for them.
-    float mx = -INFINITY;
-#pragma unroll
-    for (int c = 0; c < REG; c++) vec_max<T>(w[c], mx);
-#pragma unroll 2
-    for (int c = 0; c < LDSC; c++) vec_max<T>(staged[c * kLongThreads + tid], mx);
-    const float M = fmaxf(block_allreduce<true>(mx, slots[0]), -1e6f);
+    if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, rs.S);
+}
 
-    float sum = 0.f;
-    const float cexp = __builtin_fmaf(-M, kLog2e, kBias);
-#pragma unroll
-    for (int c = 0; c < REG; c++) { vec_sumexp<T>(w[c], cexp, sum); __builtin_amdgcn_sched_barrier(0); }
-#pragma unroll 1
-    for (int c = 0; c < LDSC; c++) vec_sumexp<T>(staged[c * kLongThreads + tid], cexp, sum);
-    const RowSum rs = make_row_sum(block_allreduce<false>(sum, slots[1]));
-    const float S = rs.S;
+// ---- forward, long rows: stream once, keep most of the row on chip ---------------------
+// 1024 lanes per row, two workgroups per CU (<= 64 VGPRs, <= 64 KiB LDS each).  Sweep 1 streams
+// the row from HBM in CHUNKS vectors per lane while each lane keeps a running maximum and the sum
+// of exponentials relative to it (rescaled when the maximum grows).  The first RK vectors of a
+// lane stay in registers and the next LK in LDS; the remaining ones are dropped.  Sweep 2 walks the
+// row backwards: the dropped vectors — the most recently fetched, so the likeliest to sit in L2
+// still — are loaded again, then the LDS and register parts follow without memory traffic.
+// Fine-grained load/compute interleaving in both sweeps lets the 32 waves of a CU hide each
+// other's latencies, which a whole-row-resident scheme with one or two workgroups per CU cannot.
+template <typename T, int CHUNKS, int RK, int LK>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void ce_forward_retain_kernel(
+    int32_t n, int32_t nvec, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
+    uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
+    constexpr int THREADS = 1024;
+    constexpr int GROUP = 2;
+    static_assert(CHUNKS % GROUP == 0 && RK % GROUP == 0 && LK % GROUP == 0, "chunk counts must be even");
+    extern __shared__ u32x4 staged[];  // LK * 1024 vectors
+    __shared__ float slots[2][THREADS / kWave];
+    const int64_t row = blockIdx.x;
+    const u32x4 *xr = (const u32x4 *)(x + row * n);
+    u32x4 *sr = (u32x4 *)(softmax + row * n);
+    const int tid = threadIdx.x;
+    const uint32_t pad = neg_inf2<T>();
+    const u32x4 pad4 = {pad, pad, pad, pad};
 
+    float m = -1e6f;   // running maximum of this lane, never below the reference's clamp
+    float s = 0.f;     // sum of 2^64 * e^(x - m) over this lane's elements so far
+    float cexp = __builtin_fmaf(-m, kLog2e, kBias);
+    // Folds GROUP vectors into (m, s).
+    auto absorb = [&](const u32x4 (&v)[GROUP]) {
+        float vm = -INFINITY;
 #pragma unroll
-    for (int c = 0; c < REG; c++) {
-        const int j = c * kLongThreads + tid;
-        if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(w[c], M, rs), sr + j);
+        for (int g = 0; g < GROUP; g++) vec_max<T>(v[g], vm);
+        if (vm > m) {
+            s *= __builtin_amdgcn_exp2f((m - vm) * kLog2e);
+            m = vm;
+            cexp = __builtin_fmaf(-m, kLog2e, kBias);
+        }
+#pragma unroll
+        for (int g = 0; g < GROUP; g++) vec_sumexp<T>(v[g], cexp, s);
+    };
+    u32x4 w[RK > 0 ? RK : 1];
+    // register part
+#pragma unroll
+    for (int c0 = 0; c0 < RK; c0 += GROUP) {
+        u32x4 v[GROUP];
+#pragma unroll
+        for (int g = 0; g < GROUP; g++) {
+            const int j = (c0 + g) * THREADS + tid;
+            v[g] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
+        }
+        absorb(v);
+#pragma unroll
+        for (int g = 0; g < GROUP; g++) w[c0 + g] = v[g];
         __builtin_amdgcn_sched_barrier(0);
     }
+    // LDS part
 #pragma unroll 1
-    for (int c = 0; c < LDSC; c++) {
-        const int j = (REG + c) * kLongThreads + tid;
-        if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(staged[c * kLongThreads + tid], M, rs), sr + j);
+    for (int c0 = RK; c0 < RK + LK; c0 += GROUP) {
+        u32x4 v[GROUP];
+#pragma unroll
+        for (int g = 0; g < GROUP; g++) {
+            const int j = (c0 + g) * THREADS + tid;
+            v[g] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
+        }
+        absorb(v);
+#pragma unroll
+        for (int g = 0; g < GROUP; g++) staged[(c0 + g - RK) * THREADS + tid] = v[g];
     }
-    if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, S);
+    // dropped part: default cache policy, meant to be found in L2 again
+#pragma unroll 1
+    for (int c0 = RK + LK; c0 < CHUNKS; c0 += GROUP) {
+        u32x4 v[GROUP];
+#pragma unroll
+        for (int g = 0; g < GROUP; g++) {
+            const int j = (c0 + g) * THREADS + tid;
+            v[g] = j < nvec ? xr[j] : pad4;
+        }
+        absorb(v);
+    }
+    const float M = block_allreduce<true>(m, slots[0]);
+    s *= __builtin_amdgcn_exp2f((m - M) * kLog2e);
+    const RowSum rs = make_row_sum(block_allreduce<false>(s, slots[1]));
+
+    // dropped part, last fetched first
+#pragma unroll 1
+    for (int c0 = CHUNKS - GROUP; c0 >= RK + LK; c0 -= GROUP) {
+        u32x4 v[GROUP];
+#pragma unroll
+        for (int g = GROUP - 1; g >= 0; g--) {
+            const int j = (c0 + g) * THREADS + tid;
+            v[g] = j < nvec ? xr[j] : pad4;
+        }
+#pragma unroll
+        for (int g = GROUP - 1; g >= 0; g--) {
+            const int j = (c0 + g) * THREADS + tid;
+            if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(v[g], M, rs), sr + j);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // LDS part (each lane reads the slots it wrote itself)
+#pragma unroll 1
+    for (int c = LK - 1; c >= 0; c--) {
+        const int j = (RK + c) * THREADS + tid;
+        if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(staged[c * THREADS + tid], M, rs), sr + j);
+    }
+    // register part
+#pragma unroll
+    for (int c = RK - 1; c >= 0; c--) {
+        const int j = c * THREADS + tid;
+        if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(reread(w[c]), M, rs), sr + j);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, rs.S);
 }
 
 // ---- forward, any row length / alignment ---------------------------------------
@@ -373,15 +498,19 @@ static int flat_grid(int64_t work_items, int threads_times_unroll) {
                        (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,     \
                        ignore_index)
 
-// Dynamic LDS beyond 64 KiB has to be allowed per kernel once.
-#define BMT_CE_LONG(REG, LDSC)                                                                                     \
+#define BMT_CE_STREAM(THREADS, UNROLL)                                                                             \
+    hipLaunchKernelGGL((ce_forward_stream_kernel<T, THREADS, UNROLL>), dim3((unsigned)m), dim3(THREADS), 0, s, n, nvec, \
+                       (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,     \
+                       ignore_index)
+
+#define BMT_CE_RETAIN(CHUNKS, RK, LK)                                                                              \
     do {                                                                                                           \
-        auto kern = ce_forward_long_kernel<T, REG, LDSC>;                                                          \
-        const size_t lds = (size_t)(LDSC) * kLongThreads * sizeof(u32x4);                                          \
+        auto kern = ce_forward_retain_kernel<T, CHUNKS, RK, LK>;                                                   \
+        const size_t lds = (size_t)(LK) * 1024 * sizeof(u32x4);                                                    \
         static const hipError_t attr = hipFuncSetAttribute((const void *)kern,                                     \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);  \
         if (attr != hipSuccess) return fail((int)attr, who, attr);                                                 \
-        hipLaunchKernelGGL(kern, dim3((unsigned)m), dim3(kLongThreads), lds, s, n, nvec, (const uint16_t *)input,  \
+        hipLaunchKernelGGL(kern, dim3((unsigned)m), dim3(1024), lds, s, n, nvec, (const uint16_t *)input,          \
                            (const int32_t *)target, (uint16_t *)softmax, (float *)output, ignore_index);           \
     } while (0)
 
@@ -392,8 +521,8 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
     if (!input || !target || !softmax || !output) return fail(-1, "cross_entropy_forward launcher: null pointer");
     hipStream_t s = (hipStream_t)stream;
     const int32_t nvec = n / 8;
-    static const int force_sweep = env_int("BMT_CE_FORCE_SWEEP", 0);
-    if (!force_sweep && rows_vectorisable(n, input, softmax) && nvec <= 1024 * 16) {
+    if (rows_vectorisable(n, input, softmax)) {
+        // rows up to 32,768 elements live in the registers of their workgroup
         if (nvec <= 64) BMT_CE_ROW(64, 1, true);
         else if (nvec <= 128) BMT_CE_ROW(64, 2, true);
         else if (nvec <= 256) BMT_CE_ROW(64, 4, true);
@@ -401,9 +530,15 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
         else if (nvec <= 1024) BMT_CE_ROW(256, 4, true);
         else if (nvec <= 2048) BMT_CE_ROW(1024, 2, true);
         else if (nvec <= 4096) BMT_CE_ROW(1024, 4, true);
-        else if (nvec <= 8192) BMT_CE_ROW(1024, 8, true);
-        else if (nvec <= 12288) BMT_CE_LONG(8, 4);
-        else BMT_CE_LONG(8, 8);
+        // up to 65,536 elements: 4 vectors per lane in registers, the rest in LDS, two workgroups per CU
+        else if (nvec <= 6144) BMT_CE_RETAIN(6, 4, 2);
+        else if (nvec <= 8192) BMT_CE_RETAIN(8, 4, 4);
+        // up to 131,072 elements: 8 vectors per lane kept, the rest fetched twice
+        else if (nvec <= 10240) BMT_CE_RETAIN(10, 4, 4);
+        else if (nvec <= 12288) BMT_CE_RETAIN(12, 4, 4);
+        else if (nvec <= 14336) BMT_CE_RETAIN(14, 4, 4);
+        else if (nvec <= 16384) BMT_CE_RETAIN(16, 4, 4);
+        else BMT_CE_STREAM(1024, 2);
     } else {
         hipLaunchKernelGGL((ce_forward_sweep_kernel<T>), dim3((unsigned)m), dim3(kSweepThreads), 0, s, n,
                            (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,

@@ -32,14 +32,6 @@ int device_cu_count() {
     return cached[dev];
 }
 
-int env_int(const char *name, int fallback) {
-    const char *s = getenv(name);
-    if (!s || !*s) return fallback;
-    char *end = nullptr;
-    long v = strtol(s, &end, 10);
-    return (end && *end == '\0') ? (int)v : fallback;
-}
-
 }  // namespace bmt
 
 extern "C" int is_bf16_supported(void) { return 1; }
