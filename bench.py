@@ -50,6 +50,10 @@ def parse():
                     help="one transformer block (202,383,360 elements) and 2,048 rows: a quick functional run, "
                          "not the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="after the timed steps, run one plain device-to-device copy of the logits buffer "
+                         "(rows * classes * 2 bytes read and written) so that rocprofv3 --pmc FETCH_SIZE / "
+                         "WRITE_SIZE readings can be scaled by a transfer of known size")
     return ap.parse_args()
 
 
@@ -210,6 +214,10 @@ def main():
     wall = time.perf_counter() - t0
     assert flag.item() == 0, "synthetic gradients are finite"
     assert torch.isfinite(row_loss).all()
+
+    if args.calibrate_copy:
+        softmax.copy_(logits)
+        torch.cuda.synchronize()
 
     ms = {name: sum(ev[i].elapsed_time(ev[i + 1]) for ev in all_events) / args.steps for i, name in enumerate(names)}
     adam_gbps = ADAM_BF16_BYTES * n / (ms["adam"] * 1e-3) / 1e9

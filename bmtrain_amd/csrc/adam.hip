@@ -4,7 +4,8 @@
 // moments and the 16-bit gradient (14 B for bf16, 12 B for fp16) and writes the
 // fp32 master, the moments and the 16-bit parameter copy (14 B / 12 B).  The
 // kernel is HBM-bound; the design goal is full-width (16 B / lane) coalesced
-// accesses with several independent tiles in flight per wave.
+// accesses, all loads of a workgroup issued before its arithmetic starts, and
+// many short workgroups so that every CU always has fresh waves to issue from.
 //
 // Arithmetic (replaces csrc/cuda/adam_cuda.cu:8-72 of the reference).  The
 // expression tree is fixed — this file is compiled with -ffp-contract=off and
