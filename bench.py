@@ -161,23 +161,26 @@ def main():
         n, rows, classes = LLAMA7B_ELEMENTS, 8192, 128256
         workload = "llama7b_full_step: has_inf_nan + adam_bf16 over 6,738,415,616 elements, ce bf16 8192x128256"
 
+    # Allocation order of a training process: 16-bit parameters first, their gradients after the first
+    # backward pass, the activations of the loss (logits, softmax) with them, and the optimizer's fp32 state
+    # last, because AdamOptimizer creates it lazily inside the first step().
     gen = torch.Generator(device=dev).manual_seed(4)
+    p16 = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    grad = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    logits = torch.empty(rows, classes, dtype=torch.bfloat16, device=dev)
+    softmax = torch.empty_like(logits)
     p32 = torch.empty(n, device=dev)
     mom = torch.empty(n, device=dev)
     var = torch.empty(n, device=dev)
-    grad = torch.empty(n, dtype=torch.bfloat16, device=dev)
-    p16 = torch.empty(n, dtype=torch.bfloat16, device=dev)
     fill_normal_(p32, 0.02, gen)
     fill_normal_(mom, 1e-4, gen)
     fill_normal_(var, 1e-6, gen, absolute=True)
     fill_normal_(grad, 1e-3, gen)
     for lo in range(0, n, 1 << 28):
         p16[lo:lo + (1 << 28)].copy_(p32[lo:lo + (1 << 28)])
-    logits = torch.empty(rows, classes, dtype=torch.bfloat16, device=dev)
     fill_normal_(logits.view(-1), 3.0, gen)
     target = torch.randint(0, classes, (rows,), generator=gen, device=dev, dtype=torch.int32)
     target[torch.randperm(rows, generator=gen, device=dev)[: rows // 20]] = -100
-    softmax = torch.empty_like(logits)
     row_loss = torch.empty(rows, dtype=torch.float32, device=dev)
     valid = (target != -100).float()
     grad_output = (valid / valid.sum()).contiguous()
