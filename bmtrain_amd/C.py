@@ -43,6 +43,8 @@ _SIGNATURES = {
     "fused_sumexp_bf16_launcher": [_i32, _i32, _p, _p, _p, _p],
     "fused_softmax_inplace_fp16_launcher": [_i32, _i32, _p, _p, _p, _p],
     "fused_softmax_inplace_bf16_launcher": [_i32, _i32, _p, _p, _p, _p],
+    "grad_stats_fp16_launcher": [_i64, _p, _p, _p, _p, _p],
+    "grad_stats_bf16_launcher": [_i64, _p, _p, _p, _p, _p],
 }
 
 _lib.bmt_hip_last_error.restype = ctypes.c_char_p
@@ -80,4 +82,13 @@ def is_bf16_supported() -> int:
     return int(_lib.is_bf16_supported())
 
 
-EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["is_bf16_supported", "bmt_hip_last_error"])
+_lib.grad_stats_workspace_floats.restype = ctypes.c_int64
+_lib.grad_stats_workspace_floats.argtypes = [_i64]
+
+
+def grad_stats_workspace_floats(n: int) -> int:
+    """Number of floats of device workspace grad_stats_*_launcher needs for n elements."""
+    return int(_lib.grad_stats_workspace_floats(n))
+
+
+EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["is_bf16_supported", "bmt_hip_last_error", "grad_stats_workspace_floats"])

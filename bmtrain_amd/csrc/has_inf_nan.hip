@@ -82,6 +82,106 @@ static int scan(int64_t n, const void *g, void *out, void *stream, const char *w
     return e == hipSuccess ? 0 : fail((int)e, who, e);
 }
 
+
+// ---- gradient statistics: overflow flag and sum of squares in one pass -----------------
+// For gradient clipping the reference computes, per tensor, g.float().norm(2) (a 4-byte copy of
+// every gradient is written and read back, optim_manager.py:186-190) and, separately, the
+// overflow flag.  This kernel reads the gradient once (2 B / element) and produces both: the
+// flag as above, and per workgroup one fp32 partial sum of squares, which a second, single
+// workgroup adds up in double precision in a fixed order and accumulates into `sumsq[0]`.
+template <typename T, int UNROLL>
+__global__ __launch_bounds__(kScanThreads) void grad_stats_kernel(
+    const uint16_t *__restrict__ g, int64_t head, int64_t nvec, int64_t n, uint8_t *__restrict__ flag,
+    float *__restrict__ partials) {
+    uint32_t hit = 0;
+    float acc = 0.f;
+    const u32x4 *body = (const u32x4 *)(g + head);
+    const int64_t base = (int64_t)blockIdx.x * (kScanThreads * UNROLL) + threadIdx.x;
+    u32x4 w[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const int64_t i = base + (int64_t)u * kScanThreads;
+        if (i < nvec) w[u] = __builtin_nontemporal_load(body + i);
+        else w[u] = u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            hit |= exp_all_ones2<T>(w[u][k]);
+            const float lo = lo_f32<T>(w[u][k]), hi = hi_f32<T>(w[u][k]);
+            acc = __builtin_fmaf(lo, lo, acc);
+            acc = __builtin_fmaf(hi, hi, acc);
+        }
+    }
+    if (blockIdx.x == 0) {   // unaligned head and tail, one element per lane
+        const int64_t tail_lo = head + nvec * 8;
+        const int64_t edge = head + (n - tail_lo);
+        if ((int64_t)threadIdx.x < edge) {
+            const int64_t i = (int64_t)threadIdx.x < head ? (int64_t)threadIdx.x : tail_lo + ((int64_t)threadIdx.x - head);
+            hit |= exp_all_ones2<T>((uint32_t)g[i]);
+            const float x = T::to_f32(g[i]);
+            acc = __builtin_fmaf(x, x, acc);
+        }
+    }
+    __shared__ float slots[kScanThreads / kWave];
+    __shared__ uint32_t any_wave;
+    if (threadIdx.x == 0) any_wave = 0;
+    __syncthreads();
+    if (__builtin_amdgcn_ballot_w64(hit != 0) != 0 && (threadIdx.x & (kWave - 1)) == 0) any_wave = 1;
+    const float total = block_allreduce<false>(acc, slots);   // contains a barrier
+    if (threadIdx.x == 0) {
+        partials[blockIdx.x] = total;
+        if (any_wave) __hip_atomic_store(flag, (uint8_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// One workgroup: lane t adds partials t, t + 1024, ... in double, then a fixed tree over the lanes.
+__global__ __launch_bounds__(kScanThreads) void grad_stats_finish_kernel(const float *__restrict__ partials, int64_t count,
+                                                                        double *__restrict__ sumsq) {
+    __shared__ double lanes[kScanThreads];
+    double acc = 0.0;
+    for (int64_t i = threadIdx.x; i < count; i += kScanThreads) acc += (double)partials[i];
+    lanes[threadIdx.x] = acc;
+    __syncthreads();
+    for (int stride = kScanThreads / 2; stride > 0; stride >>= 1) {
+        if ((int)threadIdx.x < stride) lanes[threadIdx.x] += lanes[threadIdx.x + stride];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) sumsq[0] += lanes[0];
+}
+
+static int64_t stats_tiles(int64_t n, const void *g, int64_t *head_out, int64_t *nvec_out) {
+    const uintptr_t a = (uintptr_t)g;
+    int64_t head = (int64_t)(((16 - (a & 15u)) & 15u) / 2);
+    if (head > n) head = n;
+    const int64_t nvec = (n - head) / 8;
+    const int64_t tile = (int64_t)kScanThreads * kScanUnroll;
+    const int64_t ntiles = (nvec + tile - 1) / tile;
+    if (head_out) *head_out = head;
+    if (nvec_out) *nvec_out = nvec;
+    return ntiles < 1 ? 1 : ntiles;
+}
+
+template <typename T>
+static int grad_stats(int64_t n, const void *g, void *sumsq, void *flag, void *workspace, void *stream, const char *who) {
+    if (n <= 0) return 0;
+    if (!g || !sumsq || !flag || !workspace) return fail(-1, "grad_stats launcher: null pointer");
+    if ((uintptr_t)g & 1u) return fail(-1, "grad_stats launcher: gradient pointer is not 2-byte aligned");
+    if ((uintptr_t)sumsq & 7u) return fail(-1, "grad_stats launcher: sumsq must be 8-byte aligned");
+    int64_t head = 0, nvec = 0;
+    const int64_t grid = stats_tiles(n, g, &head, &nvec);
+    if (grid > 0x7FFFFFFF) return fail(-1, "grad_stats launcher: buffer too large for one launch");
+    hipLaunchKernelGGL((grad_stats_kernel<T, kScanUnroll>), dim3((unsigned)grid), dim3(kScanThreads), 0, (hipStream_t)stream,
+                       (const uint16_t *)g, head, nvec, n, (uint8_t *)flag, (float *)workspace);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail((int)e, who, e);
+    hipLaunchKernelGGL(grad_stats_finish_kernel, dim3(1), dim3(kScanThreads), 0, (hipStream_t)stream,
+                       (const float *)workspace, grid, (double *)sumsq);
+    e = hipGetLastError();
+    return e == hipSuccess ? 0 : fail((int)e, who, e);
+}
+
 }  // namespace bmt
 
 extern "C" int has_nan_inf_fp16_launcher(int64_t n, const void *g_fp16, void *mid, void *out, void *stream) {
@@ -91,4 +191,19 @@ extern "C" int has_nan_inf_fp16_launcher(int64_t n, const void *g_fp16, void *mi
 extern "C" int has_nan_inf_bf16_launcher(int64_t n, const void *g_bf16, void *mid, void *out, void *stream) {
     (void)mid;
     return bmt::scan<bmt::BFloat16>(n, g_bf16, out, stream, "has_nan_inf_bf16_launcher");
+}
+
+extern "C" int64_t grad_stats_workspace_floats(int64_t n) {
+    // the worst case over base alignments: no head elements, every vector in the body
+    if (n <= 0) return 1;
+    const int64_t tile = (int64_t)bmt::kScanThreads * bmt::kScanUnroll * 8;
+    return (n + tile - 1) / tile + 1;
+}
+extern "C" int grad_stats_fp16_launcher(int64_t n, const void *g_fp16, void *sumsq, void *flag, void *workspace,
+                                        void *stream) {
+    return bmt::grad_stats<bmt::Half>(n, g_fp16, sumsq, flag, workspace, stream, "grad_stats_fp16_launcher");
+}
+extern "C" int grad_stats_bf16_launcher(int64_t n, const void *g_bf16, void *sumsq, void *flag, void *workspace,
+                                        void *stream) {
+    return bmt::grad_stats<bmt::BFloat16>(n, g_bf16, sumsq, flag, workspace, stream, "grad_stats_bf16_launcher");
 }

@@ -1,3 +1,3 @@
-from .cross_entropy import FusedCrossEntropy, OpFusedCrossEntropy
+from .cross_entropy import FusedCrossEntropy, OpFusedCrossEntropy, VPFusedCrossEntropy
 
-__all__ = ["FusedCrossEntropy", "OpFusedCrossEntropy"]
+__all__ = ["FusedCrossEntropy", "OpFusedCrossEntropy", "VPFusedCrossEntropy"]

@@ -10,6 +10,7 @@ from typing import Optional
 import torch
 
 from . import _function as F
+from ..global_var import config
 
 
 class OpFusedCrossEntropy(torch.autograd.Function):
@@ -36,6 +37,57 @@ class OpFusedCrossEntropy(torch.autograd.Function):
         return (softmax, None, None)
 
 
+def _tp_all_reduce(t: torch.Tensor, op: str) -> torch.Tensor:
+    """All-reduce over the tensor-parallel group.  With a group of one (the only case this
+    single-GPU package runs) the reduction is the identity; a larger group needs the
+    distributed runtime's communicator, which is not part of this package."""
+    if config.get("tp_size", 1) == 1:
+        return t
+    raise NotImplementedError("tensor-parallel all-reduce needs the distributed runtime (tp_size > 1)")
+
+
+class VPFusedCrossEntropy(torch.autograd.Function):
+    """Vocabulary-parallel cross-entropy (bmtrain/loss/cross_entropy.py:38-106): every rank holds a
+    slice [rank * V, (rank + 1) * V) of the classes.  Row maximum, target logit and sum of
+    exponentials are combined across ranks between the local kernels ``fused_sumexp`` and
+    ``fused_softmax_inplace``; the backward pass needs no communication."""
+
+    @staticmethod
+    def forward(ctx, logits: torch.Tensor, target: torch.Tensor):
+        rank = config.get("tp_rank", 0)
+        part = logits.size(-1)
+        first, last = rank * part, (rank + 1) * part
+
+        max_logits = _tp_all_reduce(torch.max(logits, dim=-1)[0].float(), "max")
+
+        outside = (target < first) | (target >= last)          # also true for ignore_index = -100
+        local_target = (target - first).masked_fill(outside, 0)
+        logits_2d = logits.view(-1, part)
+        local_target_1d = local_target.view(-1)
+        rows = torch.arange(logits_2d.size(0), device=logits_2d.device)
+        picked = logits_2d[rows, local_target_1d].contiguous().view_as(target).float()
+        picked = picked.masked_fill(outside, 0.0)
+        picked = _tp_all_reduce(picked, "sum") - max_logits
+
+        sum_exp = _tp_all_reduce(F.fused_sumexp(logits_2d, max_logits.view(-1)), "sum") + 1e-10
+        softmax = logits_2d.clone()
+        F.fused_softmax_inplace(softmax, max_logits.view(-1), sum_exp)
+
+        loss = torch.log(sum_exp.view(picked.shape)) - picked
+        ctx.save_for_backward(softmax, outside, local_target_1d)
+        ctx.logits_shape = logits.shape
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        softmax, outside, local_target_1d = ctx.saved_tensors
+        grad_2d = softmax                                           # the gradient is built in place
+        rows = torch.arange(grad_2d.size(0), device=grad_2d.device)
+        grad_2d[rows, local_target_1d] -= (1.0 - outside.view(-1).float()).to(grad_2d.dtype)
+        grad_2d.mul_(grad_output.reshape(-1, 1))
+        return grad_2d.view(ctx.logits_shape), None
+
+
 class FusedCrossEntropy(torch.nn.Module):
     r"""Cross entropy between raw scores ``input`` of shape :math:`(N, C)` and class indices
     ``target`` of shape :math:`(N)`, like :class:`torch.nn.CrossEntropyLoss`:
@@ -54,8 +106,9 @@ class FusedCrossEntropy(torch.nn.Module):
         ignore_index: target value that contributes neither loss nor gradient.
         reduction: ``'none'`` | ``'mean'`` | ``'sum'``.
         label_smoothing: only applied to fp32 input.
-        parallel: vocabulary-parallel loss across tensor-parallel ranks; needs the
-            distributed runtime and is not available in this single-GPU package.
+        parallel: vocabulary-parallel loss (``input`` holds this rank's slice of the classes).
+            With one GPU the tensor-parallel group has one member and the result equals the
+            non-parallel loss; larger groups need the distributed runtime.
 
     Example::
 
@@ -76,16 +129,13 @@ class FusedCrossEntropy(torch.nn.Module):
 
     def forward(self, input: torch.Tensor, target: torch.Tensor) -> torch.Tensor:
         if self.parallel:
-            raise NotImplementedError(
-                "FusedCrossEntropy(parallel=True) needs tensor-parallel all-reduces, which this "
-                "single-GPU package does not provide"
-            )
-        if input.dtype == torch.float32:
+            ret = VPFusedCrossEntropy.apply(input, target.long())
+        elif input.dtype == torch.float32:
             return torch.nn.functional.cross_entropy(
                 input, target.long(), weight=self.weight, ignore_index=self.ignore_index,
                 reduction=self.reduction, label_smoothing=self.label_smoothing)
-
-        ret = OpFusedCrossEntropy.apply(input, target.int(), self.ignore_index)
+        else:
+            ret = OpFusedCrossEntropy.apply(input, target.int(), self.ignore_index)
 
         ignored = target == self.ignore_index
         if self.weight is not None:

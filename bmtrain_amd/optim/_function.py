@@ -119,3 +119,23 @@ def adam_bf16(param_fp32, param_bf16, g_bf16, m_fp32, v_fp32,
         m_fp32.data_ptr(), v_fp32.data_ptr(),
         beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2, _current_stream(),
     )
+
+
+def grad_stats(g_half: torch.Tensor, sumsq: torch.Tensor, flag: torch.Tensor) -> None:
+    """One pass over a 16-bit gradient: ``sumsq`` (float64, 1 element) += sum of squares and ``flag``
+    (uint8, 1 element) = 1 if an inf / NaN is present (left alone otherwise).  Replaces, for gradient
+    clipping, the reference's ``g.float().norm(2) ** 2`` (optim_manager.py:186-190) and folds the
+    overflow scan (optim_manager.py:9-21) into the same read of the gradient."""
+    assert g_half.is_contiguous() and g_half.is_cuda, "g_half must be contiguous and on cuda"
+    assert sumsq.is_cuda and sumsq.dtype == torch.float64 and sumsq.numel() == 1, "sumsq must be one float64 on cuda"
+    assert flag.is_cuda and flag.dtype == torch.uint8 and flag.numel() == 1, "flag must be one uint8 on cuda"
+    if g_half.dtype == torch.float16:
+        launcher = C.grad_stats_fp16_launcher
+    elif g_half.dtype == torch.bfloat16:
+        _require_bf16()
+        launcher = C.grad_stats_bf16_launcher
+    else:
+        raise ValueError(f"grad_stats not supported for dtype {g_half.dtype}")
+    n = g_half.numel()
+    workspace = torch.empty(C.grad_stats_workspace_floats(n), dtype=torch.float32, device=g_half.device)
+    launcher(n, g_half.data_ptr(), sumsq.data_ptr(), flag.data_ptr(), workspace.data_ptr(), _current_stream())

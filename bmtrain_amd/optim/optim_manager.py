@@ -11,6 +11,7 @@ import torch
 
 from ..global_var import config
 from ..loss._function import has_inf_nan
+from ._function import grad_stats
 
 
 def check_overflow(param_groups):
@@ -127,9 +128,21 @@ class OptimManager:
             total_norm = max(g.abs().max() for g in grads).detach()
         else:
             norm_type = float(norm_type)
-            acc = torch.zeros(1, dtype=torch.float32, device=grads[0].device if grads else "cuda")
+            device = grads[0].device if grads else "cuda"
+            acc = torch.zeros(1, dtype=torch.float32, device=device)
+            fused = [g for g in grads if norm_type == 2.0 and g.is_cuda and g.is_contiguous()
+                     and g.dtype in (torch.float16, torch.bfloat16)]
+            if fused:
+                # 16-bit gradients: one read of each tensor instead of an fp32 copy plus a norm
+                sumsq = torch.zeros(1, dtype=torch.float64, device=device)
+                flag = torch.zeros(1, dtype=torch.uint8, device=device)
+                for g in fused:
+                    grad_stats(g, sumsq, flag)
+                acc += sumsq.float()
+            fused_ids = {id(g) for g in fused}
             for g in grads:
-                acc += g.float().norm(norm_type) ** norm_type
+                if id(g) not in fused_ids:
+                    acc += g.float().norm(norm_type) ** norm_type
             total_norm = acc[0] ** (1.0 / norm_type)
         clip_coef = float(max_norm * scale) / (total_norm + eps)
         if clip_coef < 1:

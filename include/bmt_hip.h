@@ -140,6 +140,22 @@ BMT_API int fused_softmax_inplace_fp16_launcher(int32_t m, int32_t n, void *logi
 BMT_API int fused_softmax_inplace_bf16_launcher(int32_t m, int32_t n, void *logits, const void *max_logits,
                                         const void *sum_exp_logits, void *stream);
 
+/*
+ * grad_stats_{fp16,bf16}_launcher — no single counterpart in the reference's extension: one pass over
+ * a gradient buffer that yields both quantities OptimManager needs before a step, where the reference
+ * makes several (optim_manager.py:9-21 `check_overflow` via has_nan_inf_*_launcher, and :186-190
+ * `g.float().norm(2) ** 2` through torch, which writes and re-reads an fp32 copy of every gradient).
+ *   flag[0]  (uint8)  = 1 iff some g[i] is +-inf or NaN, else untouched (sticky, as has_nan_inf_*);
+ *   sumsq[0] (double) += sum_i g[i]^2   (accumulated, so that several tensors add into one total).
+ * workspace: float[grad_stats_workspace_floats(n)] of device memory owned by the caller; its content
+ * is overwritten.  The summation order is fixed, so equal inputs give equal bits.  n <= 0 is a no-op.
+ */
+BMT_API int64_t grad_stats_workspace_floats(int64_t n);
+BMT_API int grad_stats_fp16_launcher(int64_t n, const void *g_fp16, void *sumsq, void *flag, void *workspace,
+                             void *stream);
+BMT_API int grad_stats_bf16_launcher(int64_t n, const void *g_bf16, void *sumsq, void *flag, void *workspace,
+                             void *stream);
+
 #ifdef __cplusplus
 }
 #endif

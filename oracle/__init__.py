@@ -86,6 +86,11 @@ _softmax_inplace = {
     "bf16": _sig("oracle_fused_softmax_inplace_bf16", _i64, _i64, _p, _p, _p),
 }
 
+_sumsq = {"fp16": _lib.oracle_grad_sumsq_fp16, "bf16": _lib.oracle_grad_sumsq_bf16}
+for _fn in _sumsq.values():
+    _fn.argtypes = [_i64, _p]
+    _fn.restype = ctypes.c_double
+
 u16, f32, i32, u8 = np.uint16, np.float32, np.int32, np.uint8
 
 
@@ -120,6 +125,10 @@ def has_inf_nan(bits: np.ndarray, out: np.ndarray, dtype: str) -> None:
     """Sets out[0] = 1 iff any element is inf/NaN; otherwise leaves out alone."""
     fn = {"fp16": _inf_fp16, "bf16": _inf_bf16}[dtype]
     fn(bits.size, _ptr(bits, u16), _ptr(out, u8))
+
+
+def grad_sumsq(bits: np.ndarray, dtype: str) -> float:
+    return float(_sumsq[dtype](bits.size, _ptr(bits, u16)))
 
 
 def adam_gpu_bf16(p32, p16, g16, m, v, beta1, beta2, eps, lr, scale, wd, bc1, bc2, tree=TREE_FMA_MVP):

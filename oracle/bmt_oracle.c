@@ -436,3 +436,20 @@ void oracle_fused_softmax_inplace_fp16(int64_t m, int64_t n, uint16_t *x, const 
 void oracle_fused_softmax_inplace_bf16(int64_t m, int64_t n, uint16_t *x, const float *gmax, const float *gsum) {
     softmax_inplace(m, n, x, gmax, gsum, bf16_to_float, float_to_bf16_rne);
 }
+
+/* ------------------------------------------------------------------------- */
+/* Gradient statistics                                                         */
+/* ------------------------------------------------------------------------- */
+/* What OptimManager.clip_grad_norm accumulates per tensor for norm_type 2
+ * (optim_manager.py:186-190: `g.float().norm(2) ** 2`), i.e. sum_i g_i^2, here in
+ * double precision; the overflow flag is oracle_has_inf_nan_*. */
+double oracle_grad_sumsq_fp16(int64_t n, const uint16_t *g) {
+    double s = 0.0;
+    for (int64_t i = 0; i < n; i++) { double x = (double)half_to_float(g[i]); s += x * x; }
+    return s;
+}
+double oracle_grad_sumsq_bf16(int64_t n, const uint16_t *g) {
+    double s = 0.0;
+    for (int64_t i = 0; i < n; i++) { double x = (double)bf16_to_float(g[i]); s += x * x; }
+    return s;
+}

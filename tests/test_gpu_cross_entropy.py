@@ -254,8 +254,13 @@ def test_module_contract():
         FusedCrossEntropy(weight=torch.ones(3, device="cuda"))(x.half(), tgt)
     with pytest.raises(AssertionError):
         OpFusedCrossEntropy.apply(x.half()[0], tgt.int(), -100)
-    with pytest.raises(NotImplementedError):
-        FusedCrossEntropy(parallel=True)(x.half(), tgt)
+    import bmtrain_amd
+    bmtrain_amd.config["tp_size"] = 2
+    try:
+        with pytest.raises(NotImplementedError):
+            FusedCrossEntropy(parallel=True)(x.half(), tgt)
+    finally:
+        del bmtrain_amd.config["tp_size"]
     # backward hands back the softmax buffer itself as the gradient
     xh = x.half().requires_grad_()
     out = OpFusedCrossEntropy.apply(xh, tgt.int(), -100)
@@ -263,6 +268,26 @@ def test_module_contract():
     assert xh.grad.dtype == torch.float16 and xh.grad.shape == xh.shape
     # all targets ignored: 0 / 0
     assert torch.isnan(FusedCrossEntropy()(x.half(), torch.full((8,), -100, device="cuda")))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_vocab_parallel_loss_with_one_rank(dtype):
+    """bmtrain/loss/cross_entropy.py:38-106 with a tensor-parallel group of one: same loss and
+    gradient as the fused non-parallel path and as torch in fp32 (ignored targets included)."""
+    torch.manual_seed(7)
+    N, C = 4096, 8000
+    x = torch.randn(N, C).cuda().to(dtype)
+    tgt = torch.randint(0, C, (N,)).cuda().long()
+    tgt[::7] = -100
+    vp, fused, plain = FusedCrossEntropy(parallel=True), FusedCrossEntropy(), torch.nn.CrossEntropyLoss()
+    loss_v, grad_v = _run(x, tgt, vp)
+    loss_f, grad_f = _run(x, tgt, fused)
+    loss_p, grad_p = _run(x, tgt, plain, use_float=True)
+    assert (loss_v - loss_p).abs().item() < 1e-5 and (loss_v - loss_f).abs().item() < 1e-5
+    assert (grad_v.float() - grad_p).abs().max().item() < 1e-1
+    assert grad_v[tgt == -100].count_nonzero() == 0
+    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+    assert ((grad_v.float() - grad_f.float()).abs() <= ulp * grad_f.float().abs() + 1e-3).all()
 
 
 def test_language_model_head_shape():

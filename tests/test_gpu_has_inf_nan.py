@@ -140,3 +140,55 @@ def test_full_size_buffers(name, dtype, n):
     assert gpu_flag(sample) == oracle_flag(sample, name)
     del x
     torch.cuda.empty_cache()
+
+
+# ---- gradient statistics: overflow flag + sum of squares in one pass --------------------------
+def _stats(x, sumsq_start=0.0, flag_start=0):
+    from bmtrain_amd.optim import _function as OF
+    sumsq = torch.full((1,), sumsq_start, dtype=torch.float64, device="cuda")
+    flag = torch.full((1,), flag_start, dtype=torch.uint8, device="cuda")
+    OF.grad_stats(x, sumsq, flag)
+    return sumsq.item(), int(flag.item())
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_grad_stats_against_oracle(name, dtype):
+    gen = torch.Generator().manual_seed(5)
+    base = torch.zeros(3_000_064, dtype=dtype, device="cuda")
+    for n in (1, 2, 7, 8, 9, 1000, 16384, 16385, 100003, 3_000_000):
+        for off in (0, 1, 5):
+            x = (torch.randn(n, generator=gen) * 2).to(dtype)
+            view = base[off:off + n]
+            view.copy_(x)
+            got, flag = _stats(view)
+            want = oracle.grad_sumsq(bits16(x), name)
+            assert flag == 0 and abs(got - want) <= 1e-6 * want, (n, off, got, want)
+            # identical input, identical bits; accumulation into a running total
+            again, _ = _stats(view)
+            assert again == got
+            total, _ = _stats(view, sumsq_start=10.0)
+            assert abs(total - (10.0 + got)) <= 1e-9 * (10.0 + got)
+    x = torch.ones(5000, dtype=dtype, device="cuda")
+    assert _stats(x) == (5000.0, 0)
+    x[4321] = float("inf")
+    s, flag = _stats(x)
+    assert flag == 1 and s == float("inf")
+    assert _stats(torch.ones(10, dtype=dtype, device="cuda"), flag_start=1)[1] == 1      # sticky
+    assert _stats(x[:0], sumsq_start=2.5) == (2.5, 0)                                    # empty: no-op
+
+
+def test_clip_grad_norm_uses_one_pass_and_matches_torch():
+    import bmtrain_amd as bmt
+    torch.manual_seed(9)
+    ps = [torch.nn.Parameter(torch.randn(s, device="cuda").to(d))
+          for s, d in ((100003, torch.bfloat16), (4096, torch.bfloat16), (77, torch.float16), (50, torch.float32))]
+    manager = bmt.optim.OptimManager(loss_scale=64)
+    for p in ps:
+        p.grad = (torch.randn_like(p.float()) * 64).to(p.dtype)
+    want = torch.cat([p.grad.float().flatten() for p in ps]).norm() / 64
+    before = [p.grad.clone() for p in ps]
+    got = manager.clip_grad_norm([{"params": ps}], max_norm=1.0)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=0)
+    coef = 64.0 / (want * 64 + 1e-6)
+    for p, b in zip(ps, before):
+        torch.testing.assert_close(p.grad.float(), (b.float() * coef).to(p.dtype).float(), rtol=2e-2, atol=1e-6)

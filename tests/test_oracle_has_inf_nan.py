@@ -59,3 +59,15 @@ def test_reference_style_sweep(name, dtype):
         check(x, 1)
         x[rnd.randint(0, n - 1)] = float("-inf")
         check(x, 1)
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_grad_sumsq_against_torch(name, dtype):
+    """sum of squares in double = (g.double().norm(2)) ** 2, the quantity optim_manager.py:186-190 accumulates."""
+    gen = torch.Generator().manual_seed(3)
+    for n in (1, 7, 1000, 100003):
+        g = (torch.randn(n, generator=gen) * 3).to(dtype)
+        want = (g.double().norm(2) ** 2).item()
+        got = oracle.grad_sumsq(bits16(g), name)
+        assert abs(got - want) <= 1e-12 * max(1.0, want)
+    assert oracle.grad_sumsq(bits16(torch.tensor([3.0, 4.0]).to(dtype)), name) == 25.0
