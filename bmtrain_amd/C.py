@@ -91,4 +91,30 @@ def grad_stats_workspace_floats(n: int) -> int:
     return int(_lib.grad_stats_workspace_floats(n))
 
 
-EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["is_bf16_supported", "bmt_hip_last_error", "grad_stats_workspace_floats"])
+class AdamTensor(ctypes.Structure):
+    """`bmt_adam_tensor` of include/bmt_hip.h."""
+    _fields_ = [("param_fp32", _p), ("param_16", _p), ("grad_16", _p), ("m", _p), ("v", _p), ("n", _i64)]
+
+
+def _bind_multi(name):
+    fn = getattr(_lib, name)
+    fn.argtypes = [_i32, ctypes.POINTER(AdamTensor)] + _HYPER + [_p]
+    fn.restype = ctypes.c_int
+
+    def call(tensors, beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2, stream):
+        """tensors: sequence of (param_fp32_ptr, param_16_ptr, grad_16_ptr, m_ptr, v_ptr, n)."""
+        table = (AdamTensor * len(tensors))(*[AdamTensor(*t) for t in tensors])
+        status = fn(len(tensors), table, beta1, beta2, eps, lr, scale, weight_decay, bias_correction1,
+                    bias_correction2, stream)
+        if status != 0:
+            raise RuntimeError(f"{name} failed with status {status}: {last_error()}")
+
+    call.__name__ = name
+    return call
+
+
+adam_bf16_multi_launcher = _bind_multi("adam_bf16_multi_launcher")
+adam_fp16_multi_launcher = _bind_multi("adam_fp16_multi_launcher")
+
+EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["is_bf16_supported", "bmt_hip_last_error", "grad_stats_workspace_floats",
+                                                  "adam_bf16_multi_launcher", "adam_fp16_multi_launcher"])

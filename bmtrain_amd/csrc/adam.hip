@@ -268,6 +268,120 @@ static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16
         });
 }
 
+
+// ---- several tensors in one launch ---------------------------------------------------------
+// An optimizer steps one tensor per launch in the reference (adam.py:72-159); for models with
+// many small tensors the launches, not the bytes, set the pace.  Up to kBatch tensors that share
+// their hyper-parameters are described in the kernel argument itself (no device-side table to
+// upload): workgroup b finds its tensor by scanning the running tile counts, then works on one
+// tile of that tensor exactly as the single-tensor kernel does.  The last tile of a tensor also
+// steps the up to three elements that do not fill a 4-element group.
+constexpr int kBatch = 32;
+struct AdamBatch {
+    float *p32[kBatch];
+    uint16_t *p16[kBatch];
+    const uint16_t *g16[kBatch];
+    void *mom[kBatch];          // float * (bf16 flavour) or uint16_t * (fp16 flavour)
+    float *var[kBatch];
+    int64_t n[kBatch];
+    uint32_t first_tile[kBatch + 1];
+    int32_t count;
+};
+
+template <bool FP16>
+__global__ __launch_bounds__(kAdamThreads) void adam_multi_kernel(AdamBatch batch, AdamHyper h) {
+    const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
+    int t = 0;
+    while (t + 1 < batch.count && blockIdx.x >= batch.first_tile[t + 1]) t++;
+    const int64_t n = batch.n[t];
+    const int64_t nvec = n / 4;
+    const int64_t i = (int64_t)(blockIdx.x - batch.first_tile[t]) * kAdamThreads + threadIdx.x;
+    float *p32 = batch.p32[t];
+    float *var = batch.var[t];
+    uint16_t *p16 = batch.p16[t];
+    const uint16_t *g16 = batch.g16[t];
+    if (i < nvec) {
+        u32x2 g = ld((const u32x2 *)g16 + i);
+        f32x4 p = ld((const f32x4 *)p32 + i), v = ld((const f32x4 *)var + i), m;
+        u32x2 o;
+        if (FP16) {
+            u32x2 mh = ld((const u32x2 *)batch.mom[t] + i);
+            m = f32x4{lo_f32<Half>(mh.x), hi_f32<Half>(mh.x), lo_f32<Half>(mh.y), hi_f32<Half>(mh.y)};
+            adam_group_scaled<Half>(g, m, v, p, h, omb1, omb2, lrwd, eps_s);
+            st((u32x2 *)batch.mom[t] + i, u32x2{pack2<Half>(m.x, m.y), pack2<Half>(m.z, m.w)});
+            o = u32x2{pack2<Half>(p.x, p.y), pack2<Half>(p.z, p.w)};
+        } else {
+            m = ld((const f32x4 *)batch.mom[t] + i);
+            adam_group_unscaled<BFloat16>(g, m, v, p, h, omb1, omb2, lrwd);
+            st((f32x4 *)batch.mom[t] + i, m);
+            o = u32x2{pack2<BFloat16>(p.x, p.y), pack2<BFloat16>(p.z, p.w)};
+        }
+        st((f32x4 *)p32 + i, p); st((f32x4 *)var + i, v); st((u32x2 *)p16 + i, o);
+    } else if (i - nvec < n - nvec * 4) {   // lanes right after the last group take the leftover elements
+        const int64_t e = nvec * 4 + (i - nvec);
+        float p = p32[e], v = var[e];
+        if (FP16) {
+            uint16_t *mom = (uint16_t *)batch.mom[t];
+            float m = Half::to_f32(mom[e]);
+            adam_elem_scaled(Half::to_f32(g16[e]), m, v, p, h, omb1, omb2, lrwd, eps_s);
+            mom[e] = Half::from_f32(m); p16[e] = Half::from_f32(p);
+        } else {
+            float *mom = (float *)batch.mom[t];
+            float m = mom[e];
+            adam_elem_unscaled(BFloat16::to_f32(g16[e]), m, v, p, h, omb1, omb2, lrwd);
+            mom[e] = m; p16[e] = BFloat16::from_f32(p);
+        }
+        p32[e] = p; var[e] = v;
+    }
+}
+
+// Tiles of one tensor: its 4-element groups plus one lane per leftover element.
+static int64_t multi_tiles(int64_t n) { return (n / 4 + (n % 4) + kAdamThreads - 1) / kAdamThreads; }
+
+template <bool FP16>
+static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamHyper &h, hipStream_t s, const char *who) {
+    if (count <= 0) return 0;
+    if (!tensors) return fail(-1, "adam multi launcher: null tensor table");
+    AdamBatch batch;
+    auto flush = [&]() -> hipError_t {
+        if (batch.count == 0) return hipSuccess;
+        hipLaunchKernelGGL(adam_multi_kernel<FP16>, dim3(batch.first_tile[batch.count]), dim3(kAdamThreads), 0, s, batch, h);
+        batch.count = 0;
+        batch.first_tile[0] = 0;
+        return hipGetLastError();
+    };
+    batch.count = 0;
+    batch.first_tile[0] = 0;
+    for (int32_t k = 0; k < count; k++) {
+        const bmt_adam_tensor &t = tensors[k];
+        if (t.n <= 0) continue;
+        if (!t.param_fp32 || !t.param_16 || !t.grad_16 || !t.m || !t.v) return fail(-1, "adam multi launcher: null pointer");
+        const bool aligned = (((uintptr_t)t.param_fp32 | (uintptr_t)t.v | (FP16 ? 0 : (uintptr_t)t.m)) & 15u) == 0 &&
+                             (((uintptr_t)t.param_16 | (uintptr_t)t.grad_16 | (FP16 ? (uintptr_t)t.m : 0)) & 7u) == 0;
+        const int64_t tiles = multi_tiles(t.n);
+        if (!aligned || tiles > 0x3FFFFFFF) {
+            // tensors the batch kernel does not take (unaligned views, gigantic buffers) go alone
+            hipError_t e = FP16 ? launch_fp16(t.n, (float *)t.param_fp32, (uint16_t *)t.param_16, (const uint16_t *)t.grad_16,
+                                              (uint16_t *)t.m, (float *)t.v, h, s)
+                                : launch_bf16(t.n, (float *)t.param_fp32, (uint16_t *)t.param_16, (const uint16_t *)t.grad_16,
+                                              (float *)t.m, (float *)t.v, h, s);
+            if (e != hipSuccess) return fail((int)e, who, e);
+            continue;
+        }
+        if (batch.count == kBatch || (int64_t)batch.first_tile[batch.count] + tiles > 0x7FFFFFFF) {
+            hipError_t e = flush();
+            if (e != hipSuccess) return fail((int)e, who, e);
+        }
+        const int c = batch.count;
+        batch.p32[c] = (float *)t.param_fp32; batch.p16[c] = (uint16_t *)t.param_16; batch.g16[c] = (const uint16_t *)t.grad_16;
+        batch.mom[c] = t.m; batch.var[c] = (float *)t.v; batch.n[c] = t.n;
+        batch.first_tile[c + 1] = batch.first_tile[c] + (uint32_t)tiles;
+        batch.count = c + 1;
+    }
+    hipError_t e = flush();
+    return e == hipSuccess ? 0 : fail((int)e, who, e);
+}
+
 }  // namespace bmt
 
 using namespace bmt;
@@ -292,4 +406,17 @@ extern "C" int adam_fp16_launcher(int64_t n, void *param_fp32, void *param_fp16,
     hipError_t e = launch_fp16(n, (float *)param_fp32, (uint16_t *)param_fp16, (const uint16_t *)g_fp16,
                                   (uint16_t *)m_fp16, (float *)v_fp32, h, (hipStream_t)stream);
     return e == hipSuccess ? 0 : fail((int)e, "adam_fp16_launcher", e);
+}
+
+extern "C" int adam_bf16_multi_launcher(int32_t count, const bmt_adam_tensor *tensors, float beta1, float beta2, float eps,
+                                        float lr, float scale, float weight_decay, float bias_correction1,
+                                        float bias_correction2, void *stream) {
+    AdamHyper h{beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2};
+    return adam_multi<false>(count, tensors, h, (hipStream_t)stream, "adam_bf16_multi_launcher");
+}
+extern "C" int adam_fp16_multi_launcher(int32_t count, const bmt_adam_tensor *tensors, float beta1, float beta2, float eps,
+                                        float lr, float scale, float weight_decay, float bias_correction1,
+                                        float bias_correction2, void *stream) {
+    AdamHyper h{beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2};
+    return adam_multi<true>(count, tensors, h, (hipStream_t)stream, "adam_fp16_multi_launcher");
 }

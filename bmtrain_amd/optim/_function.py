@@ -139,3 +139,36 @@ def grad_stats(g_half: torch.Tensor, sumsq: torch.Tensor, flag: torch.Tensor) ->
     n = g_half.numel()
     workspace = torch.empty(C.grad_stats_workspace_floats(n), dtype=torch.float32, device=g_half.device)
     launcher(n, g_half.data_ptr(), sumsq.data_ptr(), flag.data_ptr(), workspace.data_ptr(), _current_stream())
+
+
+def adam_multi(tensors, beta1: float, beta2: float, eps: float, lr: float, scale: float, weight_decay: float,
+               step: int) -> None:
+    """Fused GPU step over several parameter tensors that share hyper-parameters and step count.
+
+    ``tensors`` is a list of ``(param_fp32, param_16, g_16, m, v_fp32)`` as ``adam_fp16`` / ``adam_bf16`` take
+    them, all of one 16-bit flavour.  Same arithmetic per element; the tensors travel to the device in the
+    kernel arguments of as few launches as possible instead of one launch each (adam.py:72-159)."""
+    if not tensors:
+        return
+    flavour = tensors[0][1].dtype
+    assert flavour in _SIXTEEN_BIT, "adam_multi takes float16 or bfloat16 parameters"
+    moment_dtype = torch.float16 if flavour == torch.float16 else torch.float32
+    rows = []
+    for param_fp32, param_16, g_16, m, v_fp32 in tensors:
+        named = dict(param_fp32=param_fp32, param_16=param_16, g_16=g_16, m=m, v_fp32=v_fp32)
+        for name, t in named.items():
+            assert _on_gpu(t), f"{name} must be contiguous and on cuda"
+        assert param_fp32.dtype == torch.float32 and v_fp32.dtype == torch.float32, "master and v must be float32"
+        assert param_16.dtype == flavour and g_16.dtype == flavour, "all tensors must share one 16-bit dtype"
+        assert m.dtype == moment_dtype, "first moment must be float16 for float16 parameters, else float32"
+        _same_numel("param_fp32", param_fp32, param_16=param_16, g_16=g_16, m=m, v_fp32=v_fp32)
+        rows.append((param_fp32.data_ptr(), param_16.data_ptr(), g_16.data_ptr(), m.data_ptr(), v_fp32.data_ptr(),
+                     param_fp32.numel()))
+    bias_correction1 = 1 - beta1 ** step
+    bias_correction2 = 1 - beta2 ** step
+    if flavour == torch.bfloat16:
+        _require_bf16()
+        launcher = C.adam_bf16_multi_launcher
+    else:
+        launcher = C.adam_fp16_multi_launcher
+    launcher(rows, beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2, _current_stream())

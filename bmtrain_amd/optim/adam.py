@@ -23,6 +23,11 @@ class AdamOptimizer(torch.optim.Optimizer):
         validate_hyper(lr, betas, eps, weight_decay)
         super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
         self._hold_steps = hold_steps
+        # Tensors below `batch_below` elements share launches (same arithmetic per element as one launch per
+        # tensor, which remains available by setting batch_launches to False).  Larger tensors keep a launch
+        # of their own: they stream at full rate either way, and slightly faster alone.
+        self.batch_launches = True
+        self.batch_below = 1 << 20
 
     def _on_justify_scale(self, old_scale, new_scale):
         """fp16 moments are kept as moment * loss_scale (adam.py:46-55)."""
@@ -55,6 +60,8 @@ class AdamOptimizer(torch.optim.Optimizer):
 
         for group in self.param_groups:
             beta1, beta2 = group["betas"][0], group["betas"][1]
+            # 16-bit parameters of this group that can share launches: (dtype, step, lr) -> tensors
+            batches = {}
             for p in group["params"]:
                 if p.grad is None or not p.requires_grad:
                     continue
@@ -75,9 +82,16 @@ class AdamOptimizer(torch.optim.Optimizer):
                     # ... and after the increment on the fused path (adam.py:145,155).
                     state["step"] += 1
                     lr = 0.0 if state["step"] < self._hold_steps else group["lr"]
-                    fused = F.adam_fp16 if p.dtype == torch.float16 else F.adam_bf16
-                    fused(state["_param_fp32"], p, grad, state["exp_avg"], state["exp_avg_sq"],
-                          beta1, beta2, group["eps"], lr, scale, group["weight_decay"], state["step"])
+                    if (self.batch_launches and p.numel() < self.batch_below
+                            and p.is_contiguous() and grad.is_contiguous()):
+                        batches.setdefault((p.dtype, state["step"], lr), []).append(
+                            (state["_param_fp32"], p, grad, state["exp_avg"], state["exp_avg_sq"]))
+                    else:
+                        fused = F.adam_fp16 if p.dtype == torch.float16 else F.adam_bf16
+                        fused(state["_param_fp32"], p, grad, state["exp_avg"], state["exp_avg_sq"],
+                              beta1, beta2, group["eps"], lr, scale, group["weight_decay"], state["step"])
+            for (_, step, lr), tensors in batches.items():
+                F.adam_multi(tensors, beta1, beta2, group["eps"], lr, scale, group["weight_decay"], step)
         return loss
 
     def get_avg_delta():

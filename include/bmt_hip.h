@@ -141,6 +141,28 @@ BMT_API int fused_softmax_inplace_bf16_launcher(int32_t m, int32_t n, void *logi
                                         const void *sum_exp_logits, void *stream);
 
 /*
+ * adam_{fp16,bf16}_multi_launcher — no counterpart in the reference's extension, which is called once
+ * per parameter tensor from the Python loop of AdamOptimizer.step (bmtrain/optim/adam.py:72-159).  Steps
+ * `count` tensors that share their hyper-parameters (same group, same step count) in as few launches as
+ * possible; per element the arithmetic is that of adam_{fp16,bf16}_launcher, bit for bit.
+ * `tensors` is a host array; `m` is float[n] for bf16 and half[n] for fp16.  Entries with n <= 0 are skipped.
+ */
+typedef struct bmt_adam_tensor {
+    void *param_fp32;
+    void *param_16;
+    const void *grad_16;
+    void *m;
+    void *v;
+    int64_t n;
+} bmt_adam_tensor;
+BMT_API int adam_bf16_multi_launcher(int32_t count, const bmt_adam_tensor *tensors, float beta1, float beta2, float eps,
+                             float lr, float scale, float weight_decay, float bias_correction1,
+                             float bias_correction2, void *stream);
+BMT_API int adam_fp16_multi_launcher(int32_t count, const bmt_adam_tensor *tensors, float beta1, float beta2, float eps,
+                             float lr, float scale, float weight_decay, float bias_correction1,
+                             float bias_correction2, void *stream);
+
+/*
  * grad_stats_{fp16,bf16}_launcher — no single counterpart in the reference's extension: one pass over
  * a gradient buffer that yields both quantities OptimManager needs before a step, where the reference
  * makes several (optim_manager.py:9-21 `check_overflow` via has_nan_inf_*_launcher, and :186-190

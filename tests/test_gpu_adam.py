@@ -267,3 +267,39 @@ def test_more_than_2_to_the_31_elements():
     assert torch.count_nonzero(before["v"][-(1 << 20):]) == (1 << 20)
     del before, h
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("flavour", ["bf16", "fp16"])
+def test_multi_tensor_launch_equals_per_tensor_launches(flavour):
+    """adam_multi: many tensors per launch, bit for bit what one launch per tensor produces (and hence the
+    oracle), including sizes that are not multiples of 4, more tensors than one batch holds, and a tensor
+    whose views are not vector-aligned (stepped alone)."""
+    dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
+    mdt = torch.float16 if flavour == "fp16" else torch.float32
+    gen = torch.Generator().manual_seed(12)
+    sizes = [1, 2, 3, 4, 5, 1023, 1024, 4096, 4097, 4099, 128 * 128, 1237, 65536 + 3, 7, 300001] + [257] * 40
+    single, multi = [], []
+    for k, n in enumerate(sizes):
+        p = torch.randn(n, generator=gen) * 0.02
+        m = (torch.randn(n, generator=gen) * 1e-4).to(mdt)
+        v = (torch.randn(n, generator=gen) * 1e-6).abs()
+        g = (torch.randn(n, generator=gen) * 1e-3 * 8).to(dt16)
+        def place(t, off):
+            buf = torch.zeros(t.numel() + 8, dtype=t.dtype, device="cuda")
+            buf[off:off + t.numel()] = t.cuda()
+            return buf[off:off + t.numel()]
+        off = 1 if k == 9 else 0          # one unaligned tensor
+        for dest in (single, multi):
+            dest.append((place(p, off), place(torch.zeros(n, dtype=dt16), off), place(g, off), place(m, off), place(v, off)))
+    fn = F.adam_fp16 if flavour == "fp16" else F.adam_bf16
+    for step in (1, 2):
+        for p32, p16, g, m, v in single:
+            fn(p32, p16, g, m, v, 0.9, 0.999, 1e-8, 1e-3, 8.0, 0.01, step)
+        F.adam_multi(multi, 0.9, 0.999, 1e-8, 1e-3, 8.0, 0.01, step)
+    for a, b in zip(single, multi):
+        for x, y in zip(a, b):
+            assert torch.equal(x.view(torch.int16 if x.element_size() == 2 else torch.int32),
+                               y.view(torch.int16 if y.element_size() == 2 else torch.int32))
+    F.adam_multi([], 0.9, 0.999, 1e-8, 1e-3, 8.0, 0.01, 1)
+    with pytest.raises(AssertionError):
+        F.adam_multi([(single[0][0], single[0][1].float(), single[0][2], single[0][3], single[0][4])], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.0, 1)

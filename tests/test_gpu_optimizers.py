@@ -205,3 +205,24 @@ def test_constructor_validation():
     q.grad = torch.zeros_like(q)
     with pytest.raises(RuntimeError):
         bmt.optim.AdamOptimizer([q]).step()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_batched_and_per_tensor_stepping_agree_exactly(dtype):
+    torch.manual_seed(6)
+    a, b = TestModule(), TestModule()
+    state = {k: torch.randn_like(v) for k, v in a.state_dict().items()}
+    a.load_state_dict(state); b.load_state_dict(state)
+    a, b = a.cuda().to(dtype), b.cuda().to(dtype)
+    opt_a = bmt.optim.AdamOptimizer(a.parameters(), lr=1e-2, weight_decay=0.1)
+    opt_b = bmt.optim.AdamOptimizer(b.parameters(), lr=1e-2, weight_decay=0.1)
+    opt_b.batch_launches = False
+    for _ in range(5):
+        for pa, pb in zip(a.parameters(), b.parameters()):
+            g = torch.randn_like(pa)
+            pa.grad = g.clone(); pb.grad = g.clone()
+        opt_a.step(scale=2); opt_b.step(scale=2)
+    for pa, pb in zip(a.parameters(), b.parameters()):
+        assert torch.equal(pa, pb)
+        assert torch.equal(opt_a.state[pa]["_param_fp32"], opt_b.state[pb]["_param_fp32"])
+        assert torch.equal(opt_a.state[pa]["exp_avg_sq"], opt_b.state[pb]["exp_avg_sq"])
