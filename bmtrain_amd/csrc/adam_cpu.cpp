@@ -18,15 +18,22 @@
 // the CPU has them (every operation is IEEE-exact per lane, so vector and scalar code
 // agree bit for bit); the bf16 path, scalar in the reference, is vectorised as well.
 // Work is split over one thread per CPU of the calling thread's affinity mask, in
-// contiguous chunks of ceil(n / threads) elements (adam_cpu.hpp:42-80).
+// contiguous chunks of ceil(n / threads) elements (adam_cpu.hpp:42-80); the threads are kept
+// between calls instead of being created and joined every time.
 #include "../../include/bmt_hip.h"
 
 #include <immintrin.h>
 #include <sched.h>
 
+#include <pthread.h>
+
 #include <algorithm>
 #include <cmath>
+#include <condition_variable>
 #include <cstring>
+#include <functional>
+#include <mutex>
+#include <new>
 #include <thread>
 #include <vector>
 
@@ -217,20 +224,96 @@ int affinity_cpus() {
     return n > 0 ? n : 1;
 }
 
+// ---- worker threads ------------------------------------------------------------------------
+// The reference creates and joins one std::thread per chunk on every call (adam_cpu.hpp:61-75).
+// Here the helpers are created once and parked on a condition variable; the calling thread takes
+// chunk 0 itself.  The pool is rebuilt when the affinity mask asks for a different thread count
+// and is abandoned (not joined) in a forked child and at process exit, where its threads either
+// do not exist or are parked.
+class WorkerPool {
+public:
+    explicit WorkerPool(int helpers) {
+        for (int i = 0; i < helpers; i++) threads_.emplace_back([this, i] { loop(i + 1); });
+    }
+    ~WorkerPool() {
+        {
+            std::lock_guard<std::mutex> lock(mu_);
+            stop_ = true;
+            generation_++;
+        }
+        wake_.notify_all();
+        for (auto &t : threads_) t.join();
+    }
+    int helpers() const { return (int)threads_.size(); }
+
+    // Runs job(slot) for slot = 0 .. helpers(); returns when all have finished.
+    void run(const std::function<void(int)> &job) {
+        {
+            std::lock_guard<std::mutex> lock(mu_);
+            job_ = &job;
+            pending_ = (int)threads_.size();
+            generation_++;
+        }
+        wake_.notify_all();
+        job(0);
+        std::unique_lock<std::mutex> lock(mu_);
+        done_.wait(lock, [this] { return pending_ == 0; });
+        job_ = nullptr;
+    }
+
+private:
+    void loop(int slot) {
+        uint64_t seen = 0;
+        for (;;) {
+            const std::function<void(int)> *job = nullptr;
+            {
+                std::unique_lock<std::mutex> lock(mu_);
+                wake_.wait(lock, [&] { return generation_ != seen; });
+                seen = generation_;
+                if (stop_) return;
+                job = job_;
+            }
+            (*job)(slot);
+            {
+                std::lock_guard<std::mutex> lock(mu_);
+                if (--pending_ == 0) done_.notify_one();
+            }
+        }
+    }
+
+    std::vector<std::thread> threads_;
+    std::mutex mu_;
+    std::condition_variable wake_, done_;
+    const std::function<void(int)> *job_ = nullptr;
+    uint64_t generation_ = 0;
+    int pending_ = 0;
+    bool stop_ = false;
+};
+
+std::mutex g_pool_mutex;           // one fan-out at a time
+WorkerPool *g_pool = nullptr;      // leaked on purpose at exit
+void forget_pool_in_child() { g_pool = nullptr; new (&g_pool_mutex) std::mutex(); }
+
 // Runs body(lo, hi, slot) over [0, n) split into `threads` contiguous chunks of
-// ceil(n / threads) elements; slot t is private to chunk t.
+// ceil(n / threads) elements (threads = CPUs in the caller's affinity mask, adam_cpu.hpp:54-58);
+// slot t is private to chunk t.
 template <typename Body>
 void fan_out(int64_t n, const Body &body) {
     const int64_t threads = affinity_cpus();
     const int64_t chunk = std::max<int64_t>((n + threads - 1) / threads, 1);
     if (threads == 1) { body(0, n, 0); return; }
-    std::vector<std::thread> pool;
-    pool.reserve((size_t)threads);
-    for (int64_t t = 0; t < threads; t++) {
-        const int64_t lo = std::min(t * chunk, n), hi = std::min((t + 1) * chunk, n);
-        pool.emplace_back([&body, lo, hi, t] { if (lo < hi) body(lo, hi, (int)t); });
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    static const bool registered = (pthread_atfork(nullptr, nullptr, forget_pool_in_child), true);
+    (void)registered;
+    if (g_pool == nullptr || g_pool->helpers() != (int)threads - 1) {
+        delete g_pool;
+        g_pool = new WorkerPool((int)threads - 1);
     }
-    for (auto &th : pool) th.join();
+    const std::function<void(int)> job = [&](int t) {
+        const int64_t lo = std::min((int64_t)t * chunk, n), hi = std::min((int64_t)(t + 1) * chunk, n);
+        if (lo < hi) body(lo, hi, t);
+    };
+    g_pool->run(job);
 }
 
 using ChunkFn = void (*)(int64_t, int64_t, float *, uint16_t *, const uint16_t *, float *, float *, const Hyper &, Delta *);

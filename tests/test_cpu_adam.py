@@ -113,3 +113,35 @@ def test_adam_cpu_rejects_bad_arguments():
         F.adam_cpu(torch.zeros(2 * n)[::2], h, None, g, m, v, *args)
     with pytest.raises(AssertionError, match="length of 4"):
         F.adam_cpu(p, h, torch.zeros(3), g, m, v, *args)
+
+
+def test_worker_pool_survives_many_calls_affinity_changes_and_fork():
+    """The host Adam keeps its helper threads between calls: many small calls, a change of the thread count,
+    and use in a forked child must all keep working and keep matching the oracle."""
+    import multiprocessing as mp
+
+    def one_round(n, seed):
+        gen = torch.Generator().manual_seed(seed)
+        p = torch.randn(n, generator=gen) * 0.02
+        m = torch.zeros(n); v = torch.zeros(n); h = torch.zeros(n, dtype=torch.bfloat16)
+        g = torch.randn(n, generator=gen).bfloat16()
+        po, mo, vo, ho = p.numpy().copy(), m.numpy().copy(), v.numpy().copy(), np.zeros(n, np.uint16)
+        F.adam_cpu(p, h, None, g, m, v, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 1)
+        bc1, bc2 = oracle.bias_corrections(0.9, 0.999, 1)
+        oracle.adam_cpu_bf16(po, ho, None, bits16(g), mo, vo, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, bc1, bc2)
+        return np.array_equal(f32_bits(p.numpy()), f32_bits(po)) and np.array_equal(bits16(h), ho)
+
+    for k in range(200):
+        assert one_round(1 + 37 * k, k)
+    cpus = len(os.sched_getaffinity(0))
+    for threads in (2, 1, 3, cpus):
+        if threads <= cpus:
+            with affinity(threads):
+                assert one_round(10007, threads)
+    ctx = mp.get_context("fork")
+    q = ctx.Queue()
+    child = ctx.Process(target=lambda: q.put(one_round(5003, 99)))
+    child.start()
+    child.join(60)
+    assert child.exitcode == 0 and q.get(timeout=5) is True
+    assert one_round(4099, 7)
