@@ -98,9 +98,9 @@ __device__ __forceinline__ float row_loss(const uint16_t *row, int32_t n, int32_
 
 // ---- forward, register-resident row ------------------------------------------
 // One workgroup of THREADS lanes per row; lane t owns vectors t, t+THREADS, ...
-// (CHUNKS of them, 8 elements each).  KEEP_EXP: hold the 8*CHUNKS exponentials in
-// fp32 registers between the sum and the quotient; otherwise recompute them.
-template <typename T, int THREADS, int CHUNKS, bool KEEP_EXP>
+// (CHUNKS of them, 8 elements each).  The 8*CHUNKS exponentials of a lane stay in fp32
+// registers between the sum and the quotient: one exponential per element.
+template <typename T, int THREADS, int CHUNKS>
 __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
     int32_t n, int32_t nvec, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
     uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
@@ -127,26 +127,22 @@ __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
             mx = fmaxf(lo_f32<T>(w[c][k]), mx);
             mx = fmaxf(hi_f32<T>(w[c][k]), mx);
         }
-        if (!KEEP_EXP) __builtin_amdgcn_sched_barrier(0);
     }
     const float M = fmaxf(block_allreduce<true>(mx, slots[0]), -1e6f);
 
-    float e[KEEP_EXP ? CHUNKS : 1][8];
+    float e[CHUNKS][8];
     float sum = 0.f;
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            const float a = exp_biased(lo_f32<T>(w[c][k]), M), b = exp_biased(hi_f32<T>(w[c][k]), M);
-            sum += a; sum += b;
-            if (KEEP_EXP) { e[c][2 * k] = a; e[c][2 * k + 1] = b; }
+            e[c][2 * k] = exp_biased(lo_f32<T>(w[c][k]), M);
+            e[c][2 * k + 1] = exp_biased(hi_f32<T>(w[c][k]), M);
+            sum += e[c][2 * k];
+            sum += e[c][2 * k + 1];
         }
-        // Long rows live in most of the register file: keep the scheduler from overlapping
-        // the temporaries of many chunks, which would spill the row.
-        if (!KEEP_EXP) __builtin_amdgcn_sched_barrier(0);
     }
     const RowSum rs = make_row_sum(block_allreduce<false>(sum, slots[1]));
-    const float S = rs.S;
 
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
@@ -154,16 +150,11 @@ __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
         if (j < nvec) {
             u32x4 o;
 #pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const float a = KEEP_EXP ? e[c][2 * k] : exp_biased(lo_f32<T>(w[c][k]), M);
-                const float b = KEEP_EXP ? e[c][2 * k + 1] : exp_biased(hi_f32<T>(w[c][k]), M);
-                o[k] = pack2<T>(quotient(a, rs), quotient(b, rs));
-            }
+            for (int k = 0; k < 4; k++) o[k] = pack2<T>(quotient(e[c][2 * k], rs), quotient(e[c][2 * k + 1], rs));
             __builtin_nontemporal_store(o, sr + j);
         }
-        if (!KEEP_EXP) __builtin_amdgcn_sched_barrier(0);
     }
-    if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, S);
+    if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, rs.S);
 }
 
 // ---- helpers on one 16-byte vector (8 elements) ------------------------------------------
@@ -493,8 +484,8 @@ static int flat_grid(int64_t work_items, int threads_times_unroll) {
     return (int)(tiles < 1 ? 1 : (tiles < cap ? tiles : cap));
 }
 
-#define BMT_CE_ROW(THREADS, CHUNKS, KEEP)                                                                          \
-    hipLaunchKernelGGL((ce_forward_row_kernel<T, THREADS, CHUNKS, KEEP>), dim3((unsigned)m), dim3(THREADS), 0, s, n, nvec, \
+#define BMT_CE_ROW(THREADS, CHUNKS)                                                                                \
+    hipLaunchKernelGGL((ce_forward_row_kernel<T, THREADS, CHUNKS>), dim3((unsigned)m), dim3(THREADS), 0, s, n, nvec,   \
                        (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,     \
                        ignore_index)
 
@@ -523,13 +514,13 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
     const int32_t nvec = n / 8;
     if (rows_vectorisable(n, input, softmax)) {
         // rows up to 32,768 elements live in the registers of their workgroup
-        if (nvec <= 64) BMT_CE_ROW(64, 1, true);
-        else if (nvec <= 128) BMT_CE_ROW(64, 2, true);
-        else if (nvec <= 256) BMT_CE_ROW(64, 4, true);
-        else if (nvec <= 512) BMT_CE_ROW(256, 2, true);
-        else if (nvec <= 1024) BMT_CE_ROW(256, 4, true);
-        else if (nvec <= 2048) BMT_CE_ROW(1024, 2, true);
-        else if (nvec <= 4096) BMT_CE_ROW(1024, 4, true);
+        if (nvec <= 64) BMT_CE_ROW(64, 1);
+        else if (nvec <= 128) BMT_CE_ROW(64, 2);
+        else if (nvec <= 256) BMT_CE_ROW(64, 4);
+        else if (nvec <= 512) BMT_CE_ROW(256, 2);
+        else if (nvec <= 1024) BMT_CE_ROW(256, 4);
+        else if (nvec <= 2048) BMT_CE_ROW(1024, 2);
+        else if (nvec <= 4096) BMT_CE_ROW(1024, 4);
         // up to 65,536 elements: 4 vectors per lane in registers, the rest in LDS, two workgroups per CU
         else if (nvec <= 6144) BMT_CE_RETAIN(6, 4, 2);
         else if (nvec <= 8192) BMT_CE_RETAIN(8, 4, 4);
