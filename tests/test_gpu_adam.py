@@ -303,3 +303,59 @@ def test_multi_tensor_launch_equals_per_tensor_launches(flavour):
     F.adam_multi([], 0.9, 0.999, 1e-8, 1e-3, 8.0, 0.01, 1)
     with pytest.raises(AssertionError):
         F.adam_multi([(single[0][0], single[0][1].float(), single[0][2], single[0][3], single[0][4])], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.0, 1)
+
+
+def _checksum(t, chunk=1 << 28):
+    """Order-independent 64-bit checksum of a tensor's bit patterns."""
+    view = t.view(torch.int32 if t.element_size() == 4 else torch.int16)
+    total = 0
+    for lo in range(0, view.numel(), chunk):
+        total += int(view[lo:lo + chunk].to(torch.int64).sum().item())
+    return total & ((1 << 64) - 1)
+
+
+def test_whole_model_flat_buffer_equals_tensor_list():
+    """6,738,415,616 elements (a 7B-parameter model's state, 108 GB): one launch over the flat buffers.
+    Seeded slices — the first and last elements, and a stretch across element 2^32 — are checked against
+    the oracle bit for bit; then the identical inputs are stepped tensor by tensor (291 tensors of the
+    Llama-7B shapes, one launch each) and every output buffer must have the same checksum."""
+    layer = [4096 * 4096] * 4 + [4096 * 11008] * 3 + [4096] * 2
+    shapes = [32000 * 4096] + layer * 32 + [4096, 32000 * 4096]
+    n = sum(shapes)
+    assert n == 6_738_415_616 and len(shapes) == 291
+    bufs = {"h": torch.empty(n, dtype=torch.bfloat16, device="cuda"), "g": torch.empty(n, dtype=torch.bfloat16, device="cuda"),
+            "p": torch.empty(n, device="cuda"), "m": torch.empty(n, device="cuda"), "v": torch.empty(n, device="cuda")}
+
+    def fill():
+        gen = torch.Generator(device="cuda").manual_seed(4)
+        _fill_(bufs["p"], 0.02, gen); _fill_(bufs["m"], 1e-4, gen); _fill_(bufs["v"], 1e-6, gen, absolute=True)
+        _fill_(bufs["g"], 1e-3, gen)
+        bufs["h"].zero_()
+
+    fill()
+    rnd = np.random.default_rng(4)
+    starts = [0, n - 70000, (1 << 32) - 30000] + [int(s) for s in rnd.integers(0, n - 70000, 5)]
+    slices = [(s, s + 65536 + 7) for s in starts]
+    snap = {k: {s: bufs[k][s[0]:s[1]].clone() for s in slices} for k in ("p", "m", "v", "g")}
+    F.adam_bf16(bufs["p"], bufs["h"], bufs["g"], bufs["m"], bufs["v"], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100)
+    bc1, bc2 = oracle.bias_corrections(0.9, 0.999, 100)
+    for s in slices:
+        po, mo, vo = (snap[k][s].cpu().numpy().copy() for k in ("p", "m", "v"))
+        ho = np.zeros(s[1] - s[0], np.uint16)
+        oracle.adam_gpu_bf16(po, ho, bits16(snap["g"][s]), mo, vo, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, bc1, bc2)
+        assert np.array_equal(f32_bits(bufs["p"][s[0]:s[1]].cpu().numpy()), f32_bits(po)), s
+        assert np.array_equal(f32_bits(bufs["m"][s[0]:s[1]].cpu().numpy()), f32_bits(mo)), s
+        assert np.array_equal(f32_bits(bufs["v"][s[0]:s[1]].cpu().numpy()), f32_bits(vo)), s
+        assert np.array_equal(bits16(bufs["h"][s[0]:s[1]]), ho), s
+    flat = {k: _checksum(bufs[k]) for k in ("p", "m", "v", "h")}
+
+    fill()
+    lo = 0
+    for size in shapes:
+        hi = lo + size
+        F.adam_bf16(bufs["p"][lo:hi], bufs["h"][lo:hi], bufs["g"][lo:hi], bufs["m"][lo:hi], bufs["v"][lo:hi],
+                    0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100)
+        lo = hi
+    assert {k: _checksum(bufs[k]) for k in ("p", "m", "v", "h")} == flat
+    bufs.clear()
+    torch.cuda.empty_cache()

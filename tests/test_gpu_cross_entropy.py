@@ -290,13 +290,13 @@ def test_vocab_parallel_loss_with_one_rank(dtype):
     assert ((grad_v.float() - grad_f.float()).abs() <= ulp * grad_f.float().abs() + 1e-3).all()
 
 
-def test_language_model_head_shape():
-    """16,384 rows x 32,000 classes fp16, 10 % ignored, mean reduction.  Seeded rows are checked
-    against the oracle; all rows are checked through row sums, the loss against torch in fp32 on
-    the GPU, and sign / zero structure of the gradient."""
-    m, n = 16384, 32000
+@pytest.mark.parametrize("m,n,name,dtype", [(16384, 32000, "fp16", torch.float16), (8192, 128256, "bf16", torch.bfloat16)])
+def test_language_model_head_shape(m, n, name, dtype):
+    """16,384 rows x 32,000 classes fp16 and 8,192 rows x 128,256 classes bf16, 10 % ignored, mean
+    reduction.  Seeded rows are checked against the oracle; all rows are checked through row sums, the
+    loss against torch in fp32 on the GPU, and sign / zero structure of the gradient."""
     gen = torch.Generator(device="cuda").manual_seed(3)
-    x = (torch.randn(m, n, generator=gen, device="cuda") * 2).half()
+    x = (torch.randn(m, n, generator=gen, device="cuda") * 2).to(dtype)
     t = torch.randint(0, n, (m,), generator=gen, device="cuda", dtype=torch.int32)
     ignored = torch.randperm(m, generator=gen, device="cuda")[: m // 10]
     t[ignored] = -100
@@ -305,7 +305,7 @@ def test_language_model_head_shape():
     F.cross_entropy_forward(m, n, x, t, softmax, out, -100)
     rows = [0, 1, m - 1] + [int(r) for r in np.random.default_rng(3).integers(0, m, 13)]
     idx = torch.tensor(rows, device="cuda")
-    want_soft, want_loss = oracle.ce_forward(bits16(x[idx]), t[idx].cpu().numpy(), -100, "fp16")
+    want_soft, want_loss = oracle.ce_forward(bits16(x[idx]), t[idx].cpu().numpy(), -100, name)
     assert ulp_distance16(bits16(softmax[idx]), want_soft).max() <= 1
     np.testing.assert_allclose(out[idx].cpu().numpy(), want_loss, rtol=2e-6, atol=2e-6)
     sums = torch.zeros(m, device="cuda")
@@ -314,7 +314,7 @@ def test_language_model_head_shape():
         sums[lo:lo + 2048] = softmax[lo:lo + 2048].float().sum(-1)
         ref[lo:lo + 2048] = torch.nn.functional.cross_entropy(x[lo:lo + 2048].float(), t[lo:lo + 2048].long(),
                                                               ignore_index=-100, reduction="none")
-    assert (sums - 1).abs().max().item() < 2e-2            # fp16 rounding of 32,000 tiny terms
+    assert (sums - 1).abs().max().item() < 2e-2            # 16-bit rounding of n tiny terms
     torch.testing.assert_close(out, ref, rtol=1e-3, atol=1e-5)
     valid = (t != -100)
     scale = 2.0 ** 20
@@ -323,7 +323,7 @@ def test_language_model_head_shape():
     F.cross_entropy_backward_inplace(m, n, v, t, softmax, -100)
     assert softmax[~valid].count_nonzero() == 0
     check_gradient_end_to_end(got_soft, bits16(softmax[idx]), want_soft, v[idx].cpu().numpy(), t[idx].cpu().numpy(),
-                              "fp16", torch.float16)
+                              name, dtype)
     tv = t[valid].long()
     at_target = softmax[valid].gather(1, tv[:, None])
     assert (at_target < 0).all()
