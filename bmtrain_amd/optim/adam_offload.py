@@ -1,9 +1,14 @@
 """Adam with optimizer state in host memory — API of bmtrain/optim/adam_offload.py.
 
-Per step: gradients are copied device -> pinned host memory asynchronously (one event
-per parameter), each parameter is updated on the host as soon as its copy has landed
-(``_function.adam_cpu`` for 16-bit parameters, torch's functional Adam for fp32), and
-the fresh 16-bit copy is sent back host -> device asynchronously.
+Per step: gradients are copied device -> pinned host memory asynchronously, each
+parameter is updated on the host as soon as its copy has landed (``_function.adam_cpu``
+for 16-bit parameters, torch's functional Adam for fp32), and the fresh 16-bit copy is
+sent back host -> device asynchronously.  16-bit tensors larger than ``chunk_elements``
+are cut into pieces with one event each, so the host step of piece k runs while piece
+k+1 is still arriving and piece k-1 is already on its way back; the pieces are disjoint
+element ranges, so the result is that of one call over the whole tensor whenever the
+vector / scalar split inside ``adam_cpu`` falls the same way (bf16 always; fp16 to
+within the two host expression trees).
 """
 import torch
 
@@ -23,13 +28,14 @@ class AdamOffloadOptimizer(torch.optim.Optimizer):
     _bmtrain_optimizer = True
 
     def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0, hold_steps=0,
-                 record_delta=False):
+                 record_delta=False, chunk_elements=1 << 22):
         validate_hyper(lr, betas, eps, weight_decay)
         self.avg_delta = 0
         self.var_delta = 0
         super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
         self._hold_steps = hold_steps
-        self._events = {}
+        self._events = []
+        self.chunk_elements = int(chunk_elements)
         self.record_delta = record_delta
         if record_delta:
             for group in self.param_groups:
@@ -74,23 +80,39 @@ class AdamOffloadOptimizer(torch.optim.Optimizer):
                 state = self.state[p]
                 if len(state) == 0:
                     state = self._init_state(p)
-                if p not in self._events:
-                    self._events[p] = torch.cuda.Event()
                 work.append((p, state, group))
 
-        # Stage every gradient on the host; each copy gets its own event.
+        # Stage every gradient on the host, piece by piece; each copy gets its own event.
         stream = torch.cuda.current_stream()
+        pieces = {}
+        used = 0
         for p, state, _ in work:
-            staging = state["_grad_fp32"] if p.dtype == torch.float32 else state["_grad_fp16"]
-            staging.copy_(p.grad, non_blocking=True)
-            stream.record_event(self._events[p])
+            if p.dtype == torch.float32:
+                bounds = [(0, p.numel())]
+                src, dst = p.grad, state["_grad_fp32"]
+            else:
+                step_size = max(self.chunk_elements, 1)
+                bounds = [(lo, min(lo + step_size, p.numel())) for lo in range(0, p.numel(), step_size)] or [(0, 0)]
+                src, dst = p.grad.view(-1), state["_grad_fp16"].view(-1)
+            mine = []
+            for lo, hi in bounds:
+                if used == len(self._events):
+                    self._events.append(torch.cuda.Event())
+                if len(bounds) == 1:
+                    dst.copy_(src, non_blocking=True)
+                else:
+                    dst[lo:hi].copy_(src[lo:hi], non_blocking=True)
+                stream.record_event(self._events[used])
+                mine.append((lo, hi, self._events[used]))
+                used += 1
+            pieces[p] = mine
 
         sum_delta = sum_sq_delta = 0.0
         total_numel = 0
         for p, state, group in work:
-            self._events[p].synchronize()
             beta1, beta2 = group["betas"][0], group["betas"][1]
             if p.dtype == torch.float32:
+                pieces[p][0][2].synchronize()
                 grad = state["_grad_fp32"].mul_(1.0 / scale)
                 if wants_maximize(group):
                     grad = -grad
@@ -102,19 +124,32 @@ class AdamOffloadOptimizer(torch.optim.Optimizer):
                 continue
 
             state["step"] += 1
-            grad = -state["_grad_fp16"] if wants_maximize(group) else state["_grad_fp16"]
             lr = 0.0 if state["step"] < self._hold_steps else group["lr"]
-            F.adam_cpu(
-                state["_param_fp32"].view(-1), state["_param_fp16"].view(-1),
-                p._delta_info if self.record_delta else None,
-                grad.view(-1), state["exp_avg"].view(-1), state["exp_avg_sq"].view(-1),
-                beta1, beta2, group["eps"], lr, scale, group["weight_decay"], state["step"],
-            )
-            total_numel += state["_param_fp16"].numel()
+            p32, p16, g16 = state["_param_fp32"].view(-1), state["_param_fp16"].view(-1), state["_grad_fp16"].view(-1)
+            m, v = state["exp_avg"].view(-1), state["exp_avg_sq"].view(-1)
+            device_p = p.view(-1)
+            part_sum = part_sq = 0.0
+            for lo, hi, event in pieces[p]:
+                event.synchronize()
+                grad = g16[lo:hi]
+                if wants_maximize(group):
+                    grad = -grad
+                F.adam_cpu(
+                    p32[lo:hi], p16[lo:hi], p._delta_info if self.record_delta else None,
+                    grad, m[lo:hi], v[lo:hi],
+                    beta1, beta2, group["eps"], lr, scale, group["weight_decay"], state["step"],
+                )
+                if self.record_delta:
+                    part_sum += p._delta_info[2].item()
+                    part_sq += p._delta_info[3].item()
+                device_p[lo:hi].copy_(p16[lo:hi], non_blocking=True)
+            total_numel += p16.numel()
             if self.record_delta:
-                sum_delta += p._delta_info[2].item()
-                sum_sq_delta += p._delta_info[3].item()
-            p.copy_(state["_param_fp16"], non_blocking=True)
+                if len(pieces[p]) > 1 and p16.numel() > 0:    # statistics of the whole tensor, as one call leaves them
+                    mean = part_sum / p16.numel()
+                    p._delta_info.copy_(torch.tensor([mean, part_sq / p16.numel() - mean * mean, part_sum, part_sq]))
+                sum_delta += part_sum
+                sum_sq_delta += part_sq
 
         if self.record_delta and total_numel > 0:
             self.avg_delta = sum_delta / total_numel

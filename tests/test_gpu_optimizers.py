@@ -88,6 +88,37 @@ def test_fused_and_offload_agree_closely(dtype):
         bmt.optim.AdamOptimizer.get_avg_delta()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_offload_in_pieces_equals_offload_in_one_call(dtype):
+    """A tensor cut into pieces (each with its own copy event) ends in the state one host call over the
+    whole tensor leaves: bit for bit for bf16; for fp16 to within the host's two expression trees
+    (which elements take the vector lanes depends on where a call's range is cut)."""
+    torch.manual_seed(3)
+    n = 1_000_003
+    whole = torch.nn.Parameter((torch.randn(n) * 0.02).cuda().to(dtype))
+    cut = torch.nn.Parameter(whole.detach().clone())
+    opt_w = bmt.optim.AdamOffloadOptimizer([whole], lr=1e-3, weight_decay=0.01, record_delta=True, chunk_elements=1 << 40)
+    opt_c = bmt.optim.AdamOffloadOptimizer([cut], lr=1e-3, weight_decay=0.01, record_delta=True, chunk_elements=300_000)
+    for _ in range(3):
+        g = (torch.randn(n, device="cuda") * 1e-3 * 8).to(dtype)
+        whole.grad = g.clone(); cut.grad = g.clone()
+        opt_w.step(scale=8); opt_c.step(scale=8)
+        torch.cuda.synchronize()
+    sw, sc = opt_w.state[whole], opt_c.state[cut]
+    assert sw["step"] == sc["step"] == 3
+    if dtype == torch.bfloat16:
+        for key in ("_param_fp32", "exp_avg", "exp_avg_sq"):
+            assert torch.equal(sw[key], sc[key]), key
+        assert torch.equal(whole.detach(), cut.detach())
+    else:
+        for key in ("_param_fp32", "exp_avg", "exp_avg_sq"):
+            torch.testing.assert_close(sc[key], sw[key], rtol=1e-6, atol=1e-9)
+        assert ((whole.detach().float() - cut.detach().float()).abs() <= whole.detach().float().abs() * 2.0 ** -10).all()
+    assert abs(opt_c.get_avg_delta() - opt_w.get_avg_delta()) <= 1e-5 * abs(opt_w.get_avg_delta()) + 1e-9
+    assert abs(opt_c.get_var_delta() - opt_w.get_var_delta()) <= 1e-4 * opt_w.get_var_delta()
+    torch.testing.assert_close(cut._delta_info, whole._delta_info, rtol=1e-4, atol=1e-7)
+
+
 def test_overflow_skips_the_step_and_halves_the_scale():
     torch.manual_seed(2)
     p = torch.nn.Parameter(torch.randn(1000, device="cuda").half())
