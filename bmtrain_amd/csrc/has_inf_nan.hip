@@ -21,6 +21,9 @@ namespace bmt {
 // workgroups stream faster here than a resident grid that loops).
 constexpr int kScanThreads = 1024;
 constexpr int kScanUnroll = 2;
+// The statistics kernel ends in a workgroup-wide sum; a four times larger tile (128 KiB) spreads
+// that cost and keeps eight loads per lane in flight.
+constexpr int kStatsUnroll = 8;
 
 template <typename T>
 __device__ __forceinline__ uint32_t exp_all_ones2(uint32_t w) {
@@ -89,6 +92,20 @@ static int scan(int64_t n, const void *g, void *out, void *stream, const char *w
 // overflow flag.  This kernel reads the gradient once (2 B / element) and produces both: the
 // flag as above, and per workgroup one fp32 partial sum of squares, which a second, single
 // workgroup adds up in double precision in a fixed order and accumulates into `sumsq[0]`.
+// acc + lo(w)^2 + hi(w)^2 in one instruction (v_dot2_f32_f16 / v_dot2_f32_bf16): the products of
+// 16-bit values are exact in fp32, so this is the unpack-and-fma sequence without the unpacking.
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+template <typename T> __device__ __forceinline__ float sumsq2(uint32_t w, float acc);
+template <> __device__ __forceinline__ float sumsq2<Half>(uint32_t w, float acc) {
+    const half2_t h = __builtin_bit_cast(half2_t, w);
+    return __builtin_amdgcn_fdot2(h, h, acc, false);
+}
+template <> __device__ __forceinline__ float sumsq2<BFloat16>(uint32_t w, float acc) {
+    const bf16x2_t h = __builtin_bit_cast(bf16x2_t, w);
+    return __builtin_amdgcn_fdot2_f32_bf16(h, h, acc, false);
+}
+
 template <typename T, int UNROLL>
 __global__ __launch_bounds__(kScanThreads) void grad_stats_kernel(
     const uint16_t *__restrict__ g, int64_t head, int64_t nvec, int64_t n, uint8_t *__restrict__ flag,
@@ -109,9 +126,7 @@ __global__ __launch_bounds__(kScanThreads) void grad_stats_kernel(
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             hit |= exp_all_ones2<T>(w[u][k]);
-            const float lo = lo_f32<T>(w[u][k]), hi = hi_f32<T>(w[u][k]);
-            acc = __builtin_fmaf(lo, lo, acc);
-            acc = __builtin_fmaf(hi, hi, acc);
+            acc = sumsq2<T>(w[u][k], acc);
         }
     }
     if (blockIdx.x == 0) {   // unaligned head and tail, one element per lane
@@ -156,7 +171,7 @@ static int64_t stats_tiles(int64_t n, const void *g, int64_t *head_out, int64_t 
     int64_t head = (int64_t)(((16 - (a & 15u)) & 15u) / 2);
     if (head > n) head = n;
     const int64_t nvec = (n - head) / 8;
-    const int64_t tile = (int64_t)kScanThreads * kScanUnroll;
+    const int64_t tile = (int64_t)kScanThreads * kStatsUnroll;
     const int64_t ntiles = (nvec + tile - 1) / tile;
     if (head_out) *head_out = head;
     if (nvec_out) *nvec_out = nvec;
@@ -172,7 +187,7 @@ static int grad_stats(int64_t n, const void *g, void *sumsq, void *flag, void *w
     int64_t head = 0, nvec = 0;
     const int64_t grid = stats_tiles(n, g, &head, &nvec);
     if (grid > 0x7FFFFFFF) return fail(-1, "grad_stats launcher: buffer too large for one launch");
-    hipLaunchKernelGGL((grad_stats_kernel<T, kScanUnroll>), dim3((unsigned)grid), dim3(kScanThreads), 0, (hipStream_t)stream,
+    hipLaunchKernelGGL((grad_stats_kernel<T, kStatsUnroll>), dim3((unsigned)grid), dim3(kScanThreads), 0, (hipStream_t)stream,
                        (const uint16_t *)g, head, nvec, n, (uint8_t *)flag, (float *)workspace);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail((int)e, who, e);
@@ -196,7 +211,7 @@ extern "C" int has_nan_inf_bf16_launcher(int64_t n, const void *g_bf16, void *mi
 extern "C" int64_t grad_stats_workspace_floats(int64_t n) {
     // the worst case over base alignments: no head elements, every vector in the body
     if (n <= 0) return 1;
-    const int64_t tile = (int64_t)bmt::kScanThreads * bmt::kScanUnroll * 8;
+    const int64_t tile = (int64_t)bmt::kScanThreads * bmt::kStatsUnroll * 8;
     return (n + tile - 1) / tile + 1;
 }
 extern "C" int grad_stats_fp16_launcher(int64_t n, const void *g_fp16, void *sumsq, void *flag, void *workspace,

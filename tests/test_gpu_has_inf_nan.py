@@ -177,6 +177,22 @@ def test_grad_stats_against_oracle(name, dtype):
     assert _stats(x[:0], sumsq_start=2.5) == (2.5, 0)                                    # empty: no-op
 
 
+@pytest.mark.parametrize("name,dtype", [("fp16", torch.float16), ("bf16", torch.bfloat16)])
+def test_grad_stats_counts_tiny_gradients(name, dtype):
+    """Subnormal fp16 gradients (unscaled gradients below 6e-5 are) must enter the sum of squares, and so
+    must the smallest normal values of either type, alone and mixed with ordinary values."""
+    gen = torch.Generator().manual_seed(6)
+    n = 200_003
+    if dtype == torch.float16:
+        tiny = from_bits16(torch.randint(1, 0x0400, (n,), generator=gen).numpy().astype(np.uint16), dtype)   # all subnormal
+    else:
+        tiny = (torch.randn(n, generator=gen) * 1e-18).to(dtype)     # squares near the bottom of fp32's normal range
+    for x in (tiny, torch.where(torch.arange(n) % 3 == 0, (torch.randn(n, generator=gen) * 1e-3).to(dtype), tiny)):
+        got, flag = _stats(x.cuda())
+        want = oracle.grad_sumsq(bits16(x), name)
+        assert want > 0 and flag == 0 and abs(got - want) <= 1e-6 * want, (got, want)
+
+
 def test_clip_grad_norm_uses_one_pass_and_matches_torch():
     import bmtrain_amd as bmt
     torch.manual_seed(9)
