@@ -37,54 +37,33 @@ __device__ __forceinline__ float add_tiny(float s) { return (float)((double)s + 
 // ("biased"): v_exp_f32 returns 0 for results below 2^-126, and the bias keeps everything that
 // can still matter after the division (down to 2^-190) in the normal range; the factor is
 // removed again, exactly, by the reciprocal used for the quotient.
+//
+// The forward kernels are close to ALU-bound (a v_exp_f32 costs four issue slots and every
+// element needs one or two), so the exponential is three instructions and the quotient one.
+// Errors stay far below half an ulp of the 16-bit result: about 2^-20 relative from rounding
+// (x - M) * log2(e) + 64 once, 2^-22 from v_exp_f32, 2^-23 from the reciprocal and the product.
 constexpr float kLog2e = 1.44269502162933349609375f;       // fp32 nearest to log2(e)
-constexpr float kLog2eLo = 1.925963033500011e-08f;          // log2(e) - kLog2e
-constexpr float kLn2 = 0.693147182464599609375f;
 constexpr float kBias = 64.0f;
-constexpr float kTwoPowBias = 18446744073709551616.0f;      // 2^64
 constexpr float kTwoPowMinusBias = 5.42101086242752217e-20f;  // 2^-64
 
-// 2^64 * e^(x - M), accurate to about 1.5 fp32 ulp: the product (x - M) * log2(e) is carried in
-// two floats (the rounding error of the product and the low part of log2(e)), and the low part
-// enters through e^lo ~ 1 + lo.  When x - M is -inf, or so negative that the product overflows,
-// the error term is NaN or inf while the result must be 0; v_med3_f32 maps both to a finite
-// value (with a NaN operand it returns the minimum of the others), and 0 * finite = 0.  A NaN
-// argument still yields NaN through v_exp_f32.
+// 2^64 * e^(x - M).  The difference is formed first (folding M into the constant would save an
+// instruction, but rounds 64 - M * log2(e) to an error that grows with |M| and overflows for huge
+// M); x = -inf gives 0, NaN gives NaN.
 __device__ __forceinline__ float exp_biased(float x, float M) {
-    const float d = x - M;
-    const float t = d * kLog2e;
-    float lo = __builtin_fmaf(d, kLog2e, -t);
-    lo = __builtin_fmaf(d, kLog2eLo, lo);
-    lo = __builtin_amdgcn_fmed3f(lo, -1.0f, 1.0f);
-    const float e = __builtin_amdgcn_exp2f(t + kBias);
-    return __builtin_fmaf(e, lo * kLn2, e);
+    return __builtin_amdgcn_exp2f(__builtin_fmaf(x - M, kLog2e, kBias));
 }
-// Same quantity from one fma and one v_exp_f32 (relative error up to about 2^-19); used only
-// where the values are summed.  `c` = 64 - M * log2(e).
-__device__ __forceinline__ float exp_biased_fast(float x, float c) {
-    return __builtin_amdgcn_exp2f(__builtin_fmaf(x, kLog2e, c));
-}
-
-// The row's divisor in the three forms the kernels need.
+// The row's divisor in the two forms the kernels need.
 struct RowSum {
     float S;      // sum of exponentials + 1e-10, unbiased (for the loss)
-    float S64;    // S * 2^64: the divisor of the biased exponentials
-    float r64;    // correctly rounded 1 / S64
+    float r64;    // 2^-64 / S: multiplying a biased exponential by it gives the softmax value
 };
 __device__ __forceinline__ RowSum make_row_sum(float biased_sum) {
     RowSum rs;
     rs.S = add_tiny(biased_sum * kTwoPowMinusBias);
-    rs.S64 = rs.S * kTwoPowBias;
     rs.r64 = (1.0f / rs.S) * kTwoPowMinusBias;
     return rs;
 }
-// e / S, correctly rounded, from the reciprocal: one Newton correction of the product with the
-// exact remainder (Markstein); equal to the IEEE quotient the reference computes.
-__device__ __forceinline__ float quotient(float e_biased, const RowSum &rs) {
-    const float q = e_biased * rs.r64;
-    const float rem = __builtin_fmaf(-q, rs.S64, e_biased);
-    return __builtin_fmaf(rem, rs.r64, q);
-}
+__device__ __forceinline__ float quotient(float e_biased, const RowSum &rs) { return e_biased * rs.r64; }
 
 // Loss of one row; an out-of-range target that is not ignore_index yields NaN instead
 // of the reference's out-of-bounds read.
@@ -119,13 +98,17 @@ __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
         else { w[c].x = pad; w[c].y = pad; w[c].z = pad; w[c].w = pad; }
     }
 
+    // Lanes past the end of the row skip the arithmetic (whole waves do, when the row is much
+    // shorter than the launch shape's capacity): these kernels are close to ALU-bound.
     float mx = -INFINITY;
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
+        if (c * THREADS + tid < nvec) {
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            mx = fmaxf(lo_f32<T>(w[c][k]), mx);
-            mx = fmaxf(hi_f32<T>(w[c][k]), mx);
+            for (int k = 0; k < 4; k++) {
+                mx = fmaxf(lo_f32<T>(w[c][k]), mx);
+                mx = fmaxf(hi_f32<T>(w[c][k]), mx);
+            }
         }
     }
     const float M = fmaxf(block_allreduce<true>(mx, slots[0]), -1e6f);
@@ -134,12 +117,17 @@ __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
     float sum = 0.f;
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
+        if (c * THREADS + tid < nvec) {
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            e[c][2 * k] = exp_biased(lo_f32<T>(w[c][k]), M);
-            e[c][2 * k + 1] = exp_biased(hi_f32<T>(w[c][k]), M);
-            sum += e[c][2 * k];
-            sum += e[c][2 * k + 1];
+            for (int k = 0; k < 4; k++) {
+                e[c][2 * k] = exp_biased(lo_f32<T>(w[c][k]), M);
+                e[c][2 * k + 1] = exp_biased(hi_f32<T>(w[c][k]), M);
+                sum += e[c][2 * k];
+                sum += e[c][2 * k + 1];
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) e[c][k] = 0.f;
         }
     }
     const RowSum rs = make_row_sum(block_allreduce<false>(sum, slots[1]));
@@ -171,9 +159,9 @@ __device__ __forceinline__ void vec_max(const u32x4 &w, float &mx) {
     for (int k = 0; k < 4; k++) { mx = fmaxf(lo_f32<T>(w[k]), mx); mx = fmaxf(hi_f32<T>(w[k]), mx); }
 }
 template <typename T>
-__device__ __forceinline__ void vec_sumexp(const u32x4 &w, float c, float &sum) {
+__device__ __forceinline__ void vec_sumexp(const u32x4 &w, float m, float &sum) {
 #pragma unroll
-    for (int k = 0; k < 4; k++) { sum += exp_biased_fast(lo_f32<T>(w[k]), c); sum += exp_biased_fast(hi_f32<T>(w[k]), c); }
+    for (int k = 0; k < 4; k++) { sum += exp_biased(lo_f32<T>(w[k]), m); sum += exp_biased(hi_f32<T>(w[k]), m); }
 }
 template <typename T>
 __device__ __forceinline__ u32x4 vec_softmax(const u32x4 &w, float M, const RowSum &rs) {
@@ -204,7 +192,6 @@ __global__ __launch_bounds__(THREADS) void ce_forward_stream_kernel(
 
     float m = -1e6f;          // running maximum of this lane, never below the reference's clamp
     float s = 0.f;            // sum of 2^64 * e^(x - m) over this lane's elements so far
-    float cexp = __builtin_fmaf(-m, kLog2e, kBias);
     for (int j0 = 0; j0 < nvec; j0 += THREADS * UNROLL) {
         u32x4 w[UNROLL];
 #pragma unroll
@@ -218,10 +205,9 @@ __global__ __launch_bounds__(THREADS) void ce_forward_stream_kernel(
         if (vm > m) {   // rare after the first steps
             s *= __builtin_amdgcn_exp2f((m - vm) * kLog2e);
             m = vm;
-            cexp = __builtin_fmaf(-m, kLog2e, kBias);
         }
 #pragma unroll
-        for (int u = 0; u < UNROLL; u++) vec_sumexp<T>(w[u], cexp, s);
+        for (int u = 0; u < UNROLL; u++) vec_sumexp<T>(w[u], m, s);
     }
     const float M = block_allreduce<true>(m, slots[0]);
     s *= __builtin_amdgcn_exp2f((m - M) * kLog2e);
@@ -270,19 +256,18 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
 
     float m = -1e6f;   // running maximum of this lane, never below the reference's clamp
     float s = 0.f;     // sum of 2^64 * e^(x - m) over this lane's elements so far
-    float cexp = __builtin_fmaf(-m, kLog2e, kBias);
     // Folds GROUP vectors into (m, s).
-    auto absorb = [&](const u32x4 (&v)[GROUP]) {
+    auto absorb = [&](const u32x4 (&v)[GROUP], int c0) {
+        if (c0 * THREADS + (tid & ~(kWave - 1)) >= nvec) return;   // this wave is past the end of the row
         float vm = -INFINITY;
 #pragma unroll
         for (int g = 0; g < GROUP; g++) vec_max<T>(v[g], vm);
         if (vm > m) {
             s *= __builtin_amdgcn_exp2f((m - vm) * kLog2e);
             m = vm;
-            cexp = __builtin_fmaf(-m, kLog2e, kBias);
         }
 #pragma unroll
-        for (int g = 0; g < GROUP; g++) vec_sumexp<T>(v[g], cexp, s);
+        for (int g = 0; g < GROUP; g++) vec_sumexp<T>(v[g], m, s);
     };
     u32x4 w[RK > 0 ? RK : 1];
     // register part
@@ -294,7 +279,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
             const int j = (c0 + g) * THREADS + tid;
             v[g] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
         }
-        absorb(v);
+        absorb(v, c0);
 #pragma unroll
         for (int g = 0; g < GROUP; g++) w[c0 + g] = v[g];
         __builtin_amdgcn_sched_barrier(0);
@@ -308,7 +293,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
             const int j = (c0 + g) * THREADS + tid;
             v[g] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
         }
-        absorb(v);
+        absorb(v, c0);
 #pragma unroll
         for (int g = 0; g < GROUP; g++) staged[(c0 + g - RK) * THREADS + tid] = v[g];
     }
@@ -321,7 +306,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
             const int j = (c0 + g) * THREADS + tid;
             v[g] = j < nvec ? xr[j] : pad4;
         }
-        absorb(v);
+        absorb(v, c0);
     }
     const float M = block_allreduce<true>(m, slots[0]);
     s *= __builtin_amdgcn_exp2f((m - M) * kLog2e);
@@ -516,13 +501,17 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
         // rows up to 32,768 elements live in the registers of their workgroup
         if (nvec <= 64) BMT_CE_ROW(64, 1);
         else if (nvec <= 128) BMT_CE_ROW(64, 2);
+        else if (nvec <= 192) BMT_CE_ROW(64, 3);
         else if (nvec <= 256) BMT_CE_ROW(64, 4);
         else if (nvec <= 512) BMT_CE_ROW(256, 2);
+        else if (nvec <= 768) BMT_CE_ROW(256, 3);
         else if (nvec <= 1024) BMT_CE_ROW(256, 4);
+        else if (nvec <= 1536) BMT_CE_ROW(512, 3);
         else if (nvec <= 2048) BMT_CE_ROW(1024, 2);
+        else if (nvec <= 3072) BMT_CE_ROW(1024, 3);
         else if (nvec <= 4096) BMT_CE_ROW(1024, 4);
         // up to 65,536 elements: 4 vectors per lane in registers, the rest in LDS, two workgroups per CU
-        else if (nvec <= 6144) BMT_CE_RETAIN(6, 4, 2);
+        else if (nvec <= 6144) BMT_CE_RETAIN(6, 2, 4);
         else if (nvec <= 8192) BMT_CE_RETAIN(8, 4, 4);
         // up to 131,072 elements: 8 vectors per lane kept, the rest fetched twice
         else if (nvec <= 10240) BMT_CE_RETAIN(10, 4, 4);

@@ -135,18 +135,22 @@ def test_forward_backward_chain(name, dtype, n):
 
 
 @pytest.mark.parametrize("name,dtype", DTYPES)
-def test_special_rows(name, dtype):
-    n = 64
+@pytest.mark.parametrize("n", [64, 1000, 4096, 32000, 50264, 128256, 151936, 100003])   # one width per forward kernel
+def test_special_rows(name, dtype, n):
+    huge = 60000.0 if dtype == torch.float16 else 3e38
     rows = [
         torch.full((n,), float("-inf")),                 # M clamps to -1e6, S = 1e-10
         torch.full((n,), 0.5),                           # uniform
-        torch.cat([torch.tensor([60000.0 if dtype == torch.float16 else 3e38]), torch.zeros(n - 1)]),
+        torch.cat([torch.tensor([huge]), torch.zeros(n - 1)]),
         torch.cat([torch.tensor([float("nan")]), torch.ones(n - 1)]),
         torch.cat([torch.tensor([float("inf")]), torch.ones(n - 1)]),
         torch.linspace(-30, 30, n),
+        torch.cat([torch.zeros(n - 3), torch.tensor([huge, -huge, huge])]),   # equal huge values: e^0 each
+        torch.full((n,), -huge),                         # below the clamp: all exponentials 0
+        torch.linspace(-200, 0, n),                      # results down to the subnormals of the 16-bit type
     ]
     x = torch.stack(rows).to(dtype)
-    t = torch.tensor([0, 5, 0, 3, 0, n - 1], dtype=torch.int32)
+    t = torch.tensor([0, 5, 0, 3, 0, n - 1, n - 1, 1, n - 2], dtype=torch.int32)
     softmax, loss = _forward_gpu(x, t)
     want_soft, want_loss = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
     got = from_bits16(bits16(softmax), dtype).float().numpy()
