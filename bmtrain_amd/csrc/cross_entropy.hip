@@ -14,9 +14,11 @@
 //     kept; 4 vectors per lane stay in registers and up to 4 in LDS, the remainder is fetched a
 //     second time for the output sweep (ce_forward_retain_kernel);
 //   * longer rows are streamed twice (ce_forward_stream_kernel).
-// Reductions are a wave64 butterfly followed by one LDS slot per wave.  Rows whose length is not
-// a multiple of 8 or whose base is not 16-byte aligned take a three-sweep kernel with element
-// loads (ce_forward_sweep_kernel).
+// Reductions are a wave64 butterfly followed by one LDS slot per wave.  Rows may have any length
+// and start at any 2-byte offset: each row is split into a head of fewer than 8 elements, whole
+// 16-byte vectors and a tail (RowSpan).  Only when logits and softmax sit at different offsets
+// from a 16-byte boundary does a three-sweep kernel with element loads take over
+// (ce_forward_sweep_kernel).
 //
 // Backward (reference kernels :46-60, :104-121), element-wise and in place on the
 // stored softmax: x[r, i] = to16((x[r, i] - (i == target[r])) * grad_output[r]).
@@ -75,18 +77,44 @@ __device__ __forceinline__ float row_loss(const uint16_t *row, int32_t n, int32_
     return (-T::to_f32(row[t]) + M) + logf(S);
 }
 
+// How one row splits into 16-byte vectors.  A row may start anywhere (rows of odd length start at
+// every 2-byte offset in turn): up to 7 elements before the first 16-byte boundary, whole
+// vectors, up to 7 elements after the last one.  The (at most 14) edge elements are handled by
+// the first lanes of the workgroup, one element each, next to their share of the vectors.
+struct RowSpan {
+    const uint16_t *row;   // first element of the row
+    int32_t head;          // elements before the first vector
+    int32_t nvec;          // whole vectors
+    int32_t nedge;         // head + tail elements
+    __device__ __forceinline__ int32_t edge_index(int lane) const {   // lane < nedge
+        return lane < head ? lane : head + 8 * nvec + (lane - head);
+    }
+};
+__device__ __forceinline__ RowSpan row_span(const uint16_t *x, int64_t row, int32_t n) {
+    RowSpan sp;
+    sp.row = x + row * n;
+    sp.head = (int32_t)((8u - (uint32_t)(((uintptr_t)sp.row >> 1) & 7u)) & 7u);
+    if (sp.head > n) sp.head = n;
+    sp.nvec = (n - sp.head) >> 3;
+    sp.nedge = n - 8 * sp.nvec;
+    return sp;
+}
+
 // ---- forward, register-resident row ------------------------------------------
 // One workgroup of THREADS lanes per row; lane t owns vectors t, t+THREADS, ...
 // (CHUNKS of them, 8 elements each).  The 8*CHUNKS exponentials of a lane stay in fp32
 // registers between the sum and the quotient: one exponential per element.
 template <typename T, int THREADS, int CHUNKS>
 __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
-    int32_t n, int32_t nvec, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
+    int32_t n, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
     uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
     __shared__ float slots[2][THREADS / kWave];
     const int64_t row = blockIdx.x;
-    const u32x4 *xr = (const u32x4 *)(x + row * n);
-    u32x4 *sr = (u32x4 *)(softmax + row * n);
+    const RowSpan sp = row_span(x, row, n);
+    const int32_t nvec = sp.nvec;
+    const u32x4 *xr = (const u32x4 *)(sp.row + sp.head);
+    uint16_t *srow = softmax + row * n;
+    u32x4 *sr = (u32x4 *)(srow + sp.head);
     const int tid = threadIdx.x;
 
     u32x4 w[CHUNKS];
@@ -111,10 +139,19 @@ __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
             }
         }
     }
+    float edge = -INFINITY;
+    if (tid < sp.nedge) {
+        edge = T::to_f32(sp.row[sp.edge_index(tid)]);
+        mx = fmaxf(edge, mx);
+    }
     const float M = fmaxf(block_allreduce<true>(mx, slots[0]), -1e6f);
 
     float e[CHUNKS][8];
     float sum = 0.f;
+    if (tid < sp.nedge) {
+        edge = exp_biased(edge, M);
+        sum = edge;
+    }
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
         if (c * THREADS + tid < nvec) {
@@ -142,7 +179,8 @@ __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
             __builtin_nontemporal_store(o, sr + j);
         }
     }
-    if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, rs.S);
+    if (tid < sp.nedge) srow[sp.edge_index(tid)] = T::from_f32(quotient(edge, rs));
+    if (tid == 0) out[row] = row_loss<T>(sp.row, n, target[row], ignore_index, M, rs.S);
 }
 
 // ---- helpers on one 16-byte vector (8 elements) ------------------------------------------
@@ -180,12 +218,15 @@ __device__ __forceinline__ u32x4 vec_softmax(const u32x4 &w, float M, const RowS
 // it — and writes the quotient.  THREADS lanes per row, UNROLL vectors per lane per step.
 template <typename T, int THREADS, int UNROLL>
 __global__ __launch_bounds__(THREADS) void ce_forward_stream_kernel(
-    int32_t n, int32_t nvec, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
+    int32_t n, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
     uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
     __shared__ float slots[2][THREADS / kWave];
     const int64_t row = blockIdx.x;
-    const u32x4 *xr = (const u32x4 *)(x + row * n);
-    u32x4 *sr = (u32x4 *)(softmax + row * n);
+    const RowSpan sp = row_span(x, row, n);
+    const int32_t nvec = sp.nvec;
+    const u32x4 *xr = (const u32x4 *)(sp.row + sp.head);
+    uint16_t *srow = softmax + row * n;
+    u32x4 *sr = (u32x4 *)(srow + sp.head);
     const int tid = threadIdx.x;
     const uint32_t pad = neg_inf2<T>();
     const u32x4 pad4 = {pad, pad, pad, pad};
@@ -209,9 +250,21 @@ __global__ __launch_bounds__(THREADS) void ce_forward_stream_kernel(
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) vec_sumexp<T>(w[u], m, s);
     }
+    if (tid < sp.nedge) {
+        const float edge = T::to_f32(sp.row[sp.edge_index(tid)]);
+        if (edge > m) {
+            s *= __builtin_amdgcn_exp2f((m - edge) * kLog2e);
+            m = edge;
+        }
+        s += exp_biased(edge, m);
+    }
     const float M = block_allreduce<true>(m, slots[0]);
     s *= __builtin_amdgcn_exp2f((m - M) * kLog2e);
     const RowSum rs = make_row_sum(block_allreduce<false>(s, slots[1]));
+    if (tid < sp.nedge) {
+        const int32_t i = sp.edge_index(tid);
+        srow[i] = T::from_f32(quotient(exp_biased(T::to_f32(sp.row[i]), M), rs));
+    }
 
     for (int j0 = 0; j0 < nvec; j0 += THREADS * UNROLL) {
         u32x4 w[UNROLL];
@@ -226,7 +279,7 @@ __global__ __launch_bounds__(THREADS) void ce_forward_stream_kernel(
             if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(w[u], M, rs), sr + j);
         }
     }
-    if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, rs.S);
+    if (tid == 0) out[row] = row_loss<T>(sp.row, n, target[row], ignore_index, M, rs.S);
 }
 
 // ---- forward, long rows: stream once, keep most of the row on chip ---------------------
@@ -240,7 +293,7 @@ __global__ __launch_bounds__(THREADS) void ce_forward_stream_kernel(
 // other's latencies, which a whole-row-resident scheme with one or two workgroups per CU cannot.
 template <typename T, int CHUNKS, int RK, int LK>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void ce_forward_retain_kernel(
-    int32_t n, int32_t nvec, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
+    int32_t n, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
     uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
     constexpr int THREADS = 1024;
     constexpr int GROUP = 2;
@@ -248,8 +301,11 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
     extern __shared__ u32x4 staged[];  // LK * 1024 vectors
     __shared__ float slots[2][THREADS / kWave];
     const int64_t row = blockIdx.x;
-    const u32x4 *xr = (const u32x4 *)(x + row * n);
-    u32x4 *sr = (u32x4 *)(softmax + row * n);
+    const RowSpan sp = row_span(x, row, n);
+    const int32_t nvec = sp.nvec;
+    const u32x4 *xr = (const u32x4 *)(sp.row + sp.head);
+    uint16_t *srow = softmax + row * n;
+    u32x4 *sr = (u32x4 *)(srow + sp.head);
     const int tid = threadIdx.x;
     const uint32_t pad = neg_inf2<T>();
     const u32x4 pad4 = {pad, pad, pad, pad};
@@ -308,9 +364,21 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
         }
         absorb(v, c0);
     }
+    if (tid < sp.nedge) {
+        const float edge = T::to_f32(sp.row[sp.edge_index(tid)]);
+        if (edge > m) {
+            s *= __builtin_amdgcn_exp2f((m - edge) * kLog2e);
+            m = edge;
+        }
+        s += exp_biased(edge, m);
+    }
     const float M = block_allreduce<true>(m, slots[0]);
     s *= __builtin_amdgcn_exp2f((m - M) * kLog2e);
     const RowSum rs = make_row_sum(block_allreduce<false>(s, slots[1]));
+    if (tid < sp.nedge) {
+        const int32_t i = sp.edge_index(tid);
+        srow[i] = T::from_f32(quotient(exp_biased(T::to_f32(sp.row[i]), M), rs));
+    }
 
     // dropped part, last fetched first
 #pragma unroll 1
@@ -341,7 +409,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
         if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(reread(w[c]), M, rs), sr + j);
         __builtin_amdgcn_sched_barrier(0);
     }
-    if (tid == 0) out[row] = row_loss<T>(x + row * n, n, target[row], ignore_index, M, rs.S);
+    if (tid == 0) out[row] = row_loss<T>(sp.row, n, target[row], ignore_index, M, rs.S);
 }
 
 // ---- forward, any row length / alignment ---------------------------------------
@@ -379,15 +447,20 @@ __device__ __forceinline__ float flat_elem(float s, bool is_target, float a, flo
     return expf(s - a) / b;                                 // a = max, b = sum
 }
 
-// One workgroup transforms one tile of kFlatThreads * kFlatUnroll vectors and exits.
-template <typename T, int OP>
+// One workgroup transforms one tile of kFlatThreads * kFlatUnroll vectors and exits.  The array is
+// taken as one run of m * n elements: `head` elements up to the first 16-byte boundary, total_vec
+// vectors, and a tail of fewer than 8 elements (head and tail: first lanes of workgroup 0).  With a
+// row length that is not a multiple of 8 a vector can hold the end of one row and the start of
+// the next (n >= 8: never more than two rows).  RAGGED = false promises n % 8 == 0 and head == 0.
+template <typename T, int OP, bool RAGGED>
 __global__ __launch_bounds__(kFlatThreads) void ce_flat_vec_kernel(
-    int32_t nvec, int64_t total_vec, uint16_t *__restrict__ x, const float *__restrict__ row_a,
-    const float *__restrict__ row_b, const int32_t *__restrict__ target) {
-    u32x4 *xv = (u32x4 *)x;
-    const int64_t start = (int64_t)blockIdx.x * (kFlatThreads * kFlatUnroll);
-    const int64_t row0 = start / nvec;
-    const uint32_t col0 = (uint32_t)(start - row0 * nvec);
+    int32_t n, int32_t head, int64_t total_vec, int64_t total, uint16_t *__restrict__ x,
+    const float *__restrict__ row_a, const float *__restrict__ row_b, const int32_t *__restrict__ target) {
+    u32x4 *xv = (u32x4 *)(x + head);
+    const int64_t start = (int64_t)blockIdx.x * (kFlatThreads * kFlatUnroll);   // first vector of the tile
+    const int64_t first = (int64_t)head + 8 * start;                            // its first element
+    const int64_t row0 = first / n;
+    const uint32_t col0 = (uint32_t)(first - row0 * n);
     u32x4 w[kFlatUnroll];
     bool ok[kFlatUnroll];
 #pragma unroll
@@ -400,21 +473,48 @@ __global__ __launch_bounds__(kFlatThreads) void ce_flat_vec_kernel(
     for (int u = 0; u < kFlatUnroll; u++) {
         if (!ok[u]) continue;
         const int64_t g = start + (int64_t)u * kFlatThreads + threadIdx.x;
-        const uint32_t off = col0 + (uint32_t)(u * kFlatThreads + threadIdx.x);
-        const uint32_t dr = off / (uint32_t)nvec;
+        const uint32_t off = col0 + 8u * (uint32_t)(u * kFlatThreads + threadIdx.x);
+        const uint32_t dr = off / (uint32_t)n;
         const int64_t row = row0 + dr;
-        const int32_t col = (int32_t)(off - dr * (uint32_t)nvec) * 8;
+        const int32_t col = (int32_t)(off - dr * (uint32_t)n);
         const float a = row_a[row];
         const float b = OP == 1 ? row_b[row] : 0.f;
         const int32_t tk = OP == 0 ? target[row] - col : -1;  // position of the target inside this vector
         u32x4 o;
+        if (!RAGGED || col + 8 <= n) {
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const float lo = flat_elem<T, OP>(lo_f32<T>(w[u][k]), tk == 2 * k, a, b);
-            const float hi = flat_elem<T, OP>(hi_f32<T>(w[u][k]), tk == 2 * k + 1, a, b);
-            o[k] = pack2<T>(lo, hi);
+            for (int k = 0; k < 4; k++) {
+                const float lo = flat_elem<T, OP>(lo_f32<T>(w[u][k]), tk == 2 * k, a, b);
+                const float hi = flat_elem<T, OP>(hi_f32<T>(w[u][k]), tk == 2 * k + 1, a, b);
+                o[k] = pack2<T>(lo, hi);
+            }
+        } else {   // elements from position `split` on belong to the next row
+            const int32_t split = n - col;
+            const float a1 = row_a[row + 1];
+            const float b1 = OP == 1 ? row_b[row + 1] : 0.f;
+            const int32_t tk1 = OP == 0 ? target[row + 1] + split : -1;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const bool lo_next = 2 * k >= split, hi_next = 2 * k + 1 >= split;
+                const float lo = flat_elem<T, OP>(lo_f32<T>(w[u][k]), (lo_next ? tk1 : tk) == 2 * k, lo_next ? a1 : a,
+                                                  lo_next ? b1 : b);
+                const float hi = flat_elem<T, OP>(hi_f32<T>(w[u][k]), (hi_next ? tk1 : tk) == 2 * k + 1,
+                                                  hi_next ? a1 : a, hi_next ? b1 : b);
+                o[k] = pack2<T>(lo, hi);
+            }
         }
         __builtin_nontemporal_store(o, xv + g);
+    }
+    if (RAGGED && blockIdx.x == 0) {
+        const int64_t tail_lo = (int64_t)head + 8 * total_vec;
+        const int64_t nedge = (int64_t)head + (total - tail_lo);
+        if ((int64_t)threadIdx.x < nedge) {
+            const int64_t i = (int64_t)threadIdx.x < head ? (int64_t)threadIdx.x : tail_lo + ((int64_t)threadIdx.x - head);
+            const int64_t row = i / n;
+            const int32_t col = (int32_t)(i - row * n);
+            const bool is_t = OP == 0 ? (target[row] == col) : false;
+            x[i] = T::from_f32(flat_elem<T, OP>(T::to_f32(x[i]), is_t, row_a[row], OP == 1 ? row_b[row] : 0.f));
+        }
     }
 }
 
@@ -434,33 +534,31 @@ __global__ __launch_bounds__(kFlatScalarThreads) void ce_flat_scalar_kernel(
 }
 
 // ---- row sum of exponentials given the row maximum ---------------------------------
-template <typename T, bool VEC>
+template <typename T>
 __global__ __launch_bounds__(kSweepThreads) void sumexp_kernel(int32_t n, const uint16_t *__restrict__ x,
                                                                const float *__restrict__ row_max,
                                                                float *__restrict__ row_sum) {
     __shared__ float slots[kSweepThreads / kWave];
     const int64_t row = blockIdx.x;
+    const RowSpan sp = row_span(x, row, n);
+    const u32x4 *xr = (const u32x4 *)(sp.row + sp.head);
     const float M = row_max[row];
     float sum = 0.f;
-    if (VEC) {
-        const u32x4 *xr = (const u32x4 *)(x + row * n);
-        const int nvec = n / 8;
-        for (int j = threadIdx.x; j < nvec; j += kSweepThreads) {
-            const u32x4 w = __builtin_nontemporal_load(xr + j);
+    for (int j = threadIdx.x; j < sp.nvec; j += kSweepThreads) {
+        const u32x4 w = __builtin_nontemporal_load(xr + j);
 #pragma unroll
-            for (int k = 0; k < 4; k++) { sum += expf(lo_f32<T>(w[k]) - M); sum += expf(hi_f32<T>(w[k]) - M); }
-        }
-    } else {
-        const uint16_t *xr = x + row * n;
-        for (int i = threadIdx.x; i < n; i += kSweepThreads) sum += expf(T::to_f32(xr[i]) - M);
+        for (int k = 0; k < 4; k++) { sum += expf(lo_f32<T>(w[k]) - M); sum += expf(hi_f32<T>(w[k]) - M); }
     }
+    if ((int)threadIdx.x < sp.nedge) sum += expf(T::to_f32(sp.row[sp.edge_index(threadIdx.x)]) - M);
     sum = block_allreduce<false>(sum, slots);
     if (threadIdx.x == 0) row_sum[row] = sum;
 }
 
 // ---- host side ------------------------------------------------------------------
-static bool rows_vectorisable(int32_t n, const void *a, const void *b = nullptr) {
-    return (n % 8 == 0) && (((uintptr_t)a & 15u) == 0) && (b == nullptr || ((uintptr_t)b & 15u) == 0);
+// The forward kernels move input and output rows as 16-byte vectors with one split per row, which
+// needs the two arrays to sit at the same offset from a 16-byte boundary.
+static bool same_vector_phase(const void *a, const void *b) {
+    return ((((uintptr_t)a) ^ ((uintptr_t)b)) & 15u) == 0;
 }
 
 static int flat_grid(int64_t work_items, int threads_times_unroll) {
@@ -470,12 +568,12 @@ static int flat_grid(int64_t work_items, int threads_times_unroll) {
 }
 
 #define BMT_CE_ROW(THREADS, CHUNKS)                                                                                \
-    hipLaunchKernelGGL((ce_forward_row_kernel<T, THREADS, CHUNKS>), dim3((unsigned)m), dim3(THREADS), 0, s, n, nvec,   \
+    hipLaunchKernelGGL((ce_forward_row_kernel<T, THREADS, CHUNKS>), dim3((unsigned)m), dim3(THREADS), 0, s, n,         \
                        (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,     \
                        ignore_index)
 
 #define BMT_CE_STREAM(THREADS, UNROLL)                                                                             \
-    hipLaunchKernelGGL((ce_forward_stream_kernel<T, THREADS, UNROLL>), dim3((unsigned)m), dim3(THREADS), 0, s, n, nvec, \
+    hipLaunchKernelGGL((ce_forward_stream_kernel<T, THREADS, UNROLL>), dim3((unsigned)m), dim3(THREADS), 0, s, n,       \
                        (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,     \
                        ignore_index)
 
@@ -486,7 +584,7 @@ static int flat_grid(int64_t work_items, int threads_times_unroll) {
         static const hipError_t attr = hipFuncSetAttribute((const void *)kern,                                     \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);  \
         if (attr != hipSuccess) return fail((int)attr, who, attr);                                                 \
-        hipLaunchKernelGGL(kern, dim3((unsigned)m), dim3(1024), lds, s, n, nvec, (const uint16_t *)input,          \
+        hipLaunchKernelGGL(kern, dim3((unsigned)m), dim3(1024), lds, s, n, (const uint16_t *)input,                \
                            (const int32_t *)target, (uint16_t *)softmax, (float *)output, ignore_index);           \
     } while (0)
 
@@ -496,8 +594,10 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
     if (m <= 0 || n <= 0) return 0;
     if (!input || !target || !softmax || !output) return fail(-1, "cross_entropy_forward launcher: null pointer");
     hipStream_t s = (hipStream_t)stream;
-    const int32_t nvec = n / 8;
-    if (rows_vectorisable(n, input, softmax)) {
+    if ((((uintptr_t)input | (uintptr_t)softmax) & 1u) != 0)
+        return fail(-1, "cross_entropy_forward launcher: pointer is not 2-byte aligned");
+    const int32_t nvec = n / 8;   // the most vectors a row can have
+    if (same_vector_phase(input, softmax)) {
         // rows up to 32,768 elements live in the registers of their workgroup
         if (nvec <= 64) BMT_CE_ROW(64, 1);
         else if (nvec <= 128) BMT_CE_ROW(64, 2);
@@ -534,12 +634,17 @@ static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void 
     if (m <= 0 || n <= 0) return 0;
     if (!x || !row_a || (OP == 1 && !row_b) || (OP == 0 && !target)) return fail(-1, "cross_entropy launcher: null pointer");
     hipStream_t s = (hipStream_t)stream;
-    if (rows_vectorisable(n, x)) {
-        const int32_t nvec = n / 8;
-        const int64_t total = (int64_t)m * nvec;
-        const int64_t tiles = (total + kFlatThreads * kFlatUnroll - 1) / (kFlatThreads * kFlatUnroll);
+    if (((uintptr_t)x & 1u) != 0) return fail(-1, "cross_entropy launcher: pointer is not 2-byte aligned");
+    if (n >= 8) {
+        const int64_t total = (int64_t)m * n;
+        int64_t head = (int64_t)(((16 - ((uintptr_t)x & 15u)) & 15u) / 2);
+        if (head > total) head = total;
+        const int64_t total_vec = (total - head) / 8;
+        int64_t tiles = (total_vec + kFlatThreads * kFlatUnroll - 1) / (kFlatThreads * kFlatUnroll);
+        if (tiles < 1) tiles = 1;
         if (tiles > 0x7FFFFFFF) return fail(-1, "cross_entropy launcher: tensor too large for one launch");
-        hipLaunchKernelGGL((ce_flat_vec_kernel<T, OP>), dim3((unsigned)tiles), dim3(kFlatThreads), 0, s, nvec, total,
+        auto kern = (n % 8 == 0 && head == 0) ? ce_flat_vec_kernel<T, OP, false> : ce_flat_vec_kernel<T, OP, true>;
+        hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(kFlatThreads), 0, s, n, (int32_t)head, total_vec, total,
                            (uint16_t *)x, (const float *)row_a, (const float *)row_b, (const int32_t *)target);
     } else {
         const int64_t total = (int64_t)m * n;
@@ -556,12 +661,9 @@ static int sumexp(int32_t m, int32_t n, const void *logits, const void *row_max,
     if (m <= 0 || n <= 0) return 0;
     if (!logits || !row_max || !row_sum) return fail(-1, "fused_sumexp launcher: null pointer");
     hipStream_t s = (hipStream_t)stream;
-    if (rows_vectorisable(n, logits))
-        hipLaunchKernelGGL((sumexp_kernel<T, true>), dim3((unsigned)m), dim3(kSweepThreads), 0, s, n, (const uint16_t *)logits,
-                           (const float *)row_max, (float *)row_sum);
-    else
-        hipLaunchKernelGGL((sumexp_kernel<T, false>), dim3((unsigned)m), dim3(kSweepThreads), 0, s, n, (const uint16_t *)logits,
-                           (const float *)row_max, (float *)row_sum);
+    if (((uintptr_t)logits & 1u) != 0) return fail(-1, "fused_sumexp launcher: pointer is not 2-byte aligned");
+    hipLaunchKernelGGL((sumexp_kernel<T>), dim3((unsigned)m), dim3(kSweepThreads), 0, s, n, (const uint16_t *)logits,
+                       (const float *)row_max, (float *)row_sum);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : fail((int)e, who, e);
 }

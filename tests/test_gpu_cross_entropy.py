@@ -33,10 +33,12 @@ def _forward_gpu(x, t, ignore=-100):
     return softmax, out
 
 
-# every launch shape of the forward: one wave per row, 256 and 1024 lanes per row with 1..8 vectors
-# per lane in registers, registers + LDS, and the element-load kernel (n % 8 != 0, or very long rows)
-WIDTHS = [1, 2, 3, 7, 8, 10, 16, 90, 100, 512, 520, 1000, 1024, 2048, 2056, 4096, 8192, 8200, 10240, 16384, 30000,
-          32000, 32768, 50264, 65536, 65544, 98304, 100000, 128256, 131072, 131080, 151936]
+# every launch shape of the forward: one wave per row, 256 / 512 / 1024 lanes per row with 1..4 vectors per
+# lane in registers, registers + LDS with and without a re-read part, two streaming sweeps; row lengths that
+# are not multiples of 8 (rows then start at every 2-byte offset in turn) in each of them
+WIDTHS = [1, 2, 3, 7, 8, 9, 10, 15, 16, 17, 90, 100, 512, 513, 520, 1000, 1001, 1024, 1500, 2048, 2056, 4096, 4097, 6100,
+          8192, 8200, 10240, 12288, 12295, 16384, 20001, 30000, 32000, 32001, 32768, 32775, 49151, 50257, 50264, 65535,
+          65536, 65544, 98304, 100000, 100003, 128256, 128257, 131072, 131079, 131080, 151936, 151937]
 
 
 @pytest.mark.parametrize("name,dtype", DTYPES)
@@ -55,7 +57,7 @@ def test_forward_against_oracle(name, dtype, n):
 
 
 @pytest.mark.parametrize("name,dtype", DTYPES)
-@pytest.mark.parametrize("n", [1, 5, 8, 100, 1000, 4096, 32000, 50001, 128256])
+@pytest.mark.parametrize("n", [1, 5, 7, 8, 9, 15, 100, 1000, 1001, 4096, 32000, 50001, 50257, 128256, 128257])
 def test_backward_bit_exact_on_identical_input(name, dtype, n):
     m = 11
     x, t = _case(m, n, dtype, seed=n + 1)
@@ -164,33 +166,37 @@ def test_special_rows(name, dtype, n):
 
 
 @pytest.mark.parametrize("name,dtype", DTYPES)
-def test_unaligned_row_base_takes_the_element_kernel(name, dtype):
-    m, n = 6, 1024
-    x, t = _case(m, n, dtype, seed=3)
-    buf = torch.zeros(m * n + 8, dtype=dtype, device="cuda")
-    for off in (1, 4):
+@pytest.mark.parametrize("m,n", [(6, 1024), (5, 1001), (3, 50257), (2, 131075), (40, 5), (9, 8)])
+def test_unaligned_bases(name, dtype, m, n):
+    """Arrays that start at any 2-byte offset: logits and softmax at the same offset from a 16-byte boundary
+    (vector kernels with a per-row split) and at different ones (element loads); nothing outside is written."""
+    x, t = _case(m, n, dtype, seed=n + m)
+    want_soft, want_loss = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
+    buf = torch.zeros(m * n + 16, dtype=dtype, device="cuda")
+    for off, soft_off in ((1, 1), (4, 4), (7, 7), (3, 11), (0, 8), (2, 5), (0, 1)):
         xg = buf[off:off + m * n].view(m, n)
         xg.copy_(x)
-        soft_buf = torch.zeros(m * n + 8, dtype=dtype, device="cuda")
-        soft = soft_buf[off:off + m * n].view(m, n)
+        soft_buf = torch.zeros(m * n + 16, dtype=dtype, device="cuda")
+        soft = soft_buf[soft_off:soft_off + m * n].view(m, n)
         out = torch.empty(m, dtype=torch.float32, device="cuda")
         F.cross_entropy_forward(m, n, xg, t.cuda(), soft, out, -100)
-        want_soft, want_loss = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
-        assert ulp_distance16(bits16(soft), want_soft).max() <= 1
-        assert soft_buf[:off].count_nonzero() == 0 and soft_buf[off + m * n:].count_nonzero() == 0
+        assert ulp_distance16(bits16(soft), want_soft).max() <= 1, (off, soft_off)
+        np.testing.assert_allclose(out.cpu().numpy(), want_loss, rtol=2e-6, atol=2e-6)
+        assert soft_buf[:soft_off].count_nonzero() == 0 and soft_buf[soft_off + m * n:].count_nonzero() == 0
         v = torch.rand(m)
         want = bits16(soft)
         oracle.ce_backward_inplace(v.numpy(), t.numpy(), want, -100, name)
         F.cross_entropy_backward_inplace(m, n, v.cuda(), t.cuda(), soft, -100)
-        assert np.array_equal(bits16(soft), want)
-        assert soft_buf[:off].count_nonzero() == 0 and soft_buf[off + m * n:].count_nonzero() == 0
+        assert np.array_equal(bits16(soft), want), (off, soft_off)
+        assert soft_buf[:soft_off].count_nonzero() == 0 and soft_buf[soft_off + m * n:].count_nonzero() == 0
 
 
 @pytest.mark.parametrize("name,dtype", DTYPES)
 def test_sumexp_and_softmax_inplace(name, dtype):
-    for m, n in ((5, 1000), (3, 32000), (4, 777)):
+    for m, n, off in ((5, 1000, 0), (3, 32000, 0), (4, 777, 0), (7, 50257, 3), (33, 5, 1), (2, 9, 7)):
         x, _ = _case(m, n, dtype, seed=n)
-        xg = x.cuda()
+        xg = torch.zeros(m * n + 8, dtype=dtype, device="cuda")[off:off + m * n].view(m, n)
+        xg.copy_(x)
         mx = xg.float().max(-1).values.contiguous()
         se = F.fused_sumexp(xg, mx)
         want_se = oracle.fused_sumexp(bits16(x), mx.cpu().numpy(), name)
