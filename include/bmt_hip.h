@@ -51,6 +51,8 @@ BMT_API int has_nan_inf_bf16_launcher(int64_t n, const void *g_bf16, void *mid, 
  * One fused step over n elements.  fp16 flavour: g is the loss-scaled gradient and
  * the moments are kept multiplied by `scale` (m in fp16, v in fp32).
  * Writes param_fp32, param_fp16 (round-to-nearest-even), m_fp16, v_fp32.  n <= 0: no-op.
+ * param_fp16 is output only: while a launch of 2^25 elements or more is in flight its last
+ * 8 bytes hold a tile counter, and its previous contents are never read.
  */
 BMT_API int adam_fp16_launcher(int64_t n, void *param_fp32, void *param_fp16, const void *g_fp16,
                        void *m_fp16, void *v_fp32,

@@ -244,6 +244,44 @@ def test_one_transformer_block_flat_buffer():
                            after[k].view(torch.int32 if k != "h" else torch.int16)), k
 
 
+@pytest.mark.parametrize("flavour", ["bf16", "fp16"])
+@pytest.mark.parametrize("n,off", [((1 << 25) - 4096 + 3, 0), ((1 << 25) + 12345, 0), ((1 << 25) + 4096 * 3 + 1, 2)])
+def test_around_the_launch_size_where_tiles_are_handed_out_by_ticket(flavour, n, off):
+    """From 8,192 tiles on, workgroups draw their tile from a counter kept in the last vector of the 16-bit
+    output.  Whole-buffer comparison with the oracle just below and above that size, with an unaligned head:
+    every tile stepped exactly once, and the counter's place holds its real value afterwards."""
+    dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
+    mdt = torch.float16 if flavour == "fp16" else torch.float32
+    scale = 4.0 if flavour == "fp16" else 1.0
+    gen = torch.Generator().manual_seed(n)
+    p = torch.randn(n, generator=gen) * 0.02
+    m = (torch.randn(n, generator=gen) * 1e-4 * scale).to(mdt)
+    v = (torch.randn(n, generator=gen) * 1e-6 * scale).abs()
+    g = (torch.randn(n, generator=gen) * 1e-3 * scale).to(dt16)
+    def place(t, fill=0):
+        buf = torch.full((n + 8,), fill, dtype=t.dtype, device="cuda")
+        buf[off:off + n] = t.cuda()
+        return buf[off:off + n]
+    pg, mg, vg, gg = place(p), place(m), place(v), place(g)
+    hg = place(torch.zeros(n, dtype=dt16), fill=-1)        # a non-zero pattern where the counter will live
+    fn = F.adam_fp16 if flavour == "fp16" else F.adam_bf16
+    fn(pg, hg, gg, mg, vg, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, 7)
+    bc1, bc2 = oracle.bias_corrections(0.9, 0.999, 7)
+    po, vo = p.numpy().copy(), v.numpy().copy()
+    ho = np.zeros(n, np.uint16)
+    if flavour == "fp16":
+        mo = bits16(m)
+        oracle.adam_gpu_fp16(po, ho, bits16(g), mo, vo, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, bc1, bc2)
+        assert np.array_equal(bits16(mg), mo)
+    else:
+        mo = m.numpy().copy()
+        oracle.adam_gpu_bf16(po, ho, bits16(g), mo, vo, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, bc1, bc2)
+        assert np.array_equal(f32_bits(mg.cpu().numpy()), f32_bits(mo))
+    assert np.array_equal(f32_bits(pg.cpu().numpy()), f32_bits(po))
+    assert np.array_equal(f32_bits(vg.cpu().numpy()), f32_bits(vo))
+    assert np.array_equal(bits16(hg), ho)
+
+
 def test_more_than_2_to_the_31_elements():
     """Element counts beyond int32 (the reference's launcher takes `int n`): the last stretch of a
     2^31 + 12345 element buffer must be stepped, and stepped correctly."""
