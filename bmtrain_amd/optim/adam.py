@@ -1,8 +1,11 @@
 """On-device Adam for fp32 / fp16 / bf16 parameters — API of bmtrain/optim/adam.py.
 
-16-bit parameters take one fused HIP launch per tensor (``_function.adam_fp16`` /
+16-bit parameters are stepped by fused HIP launches (``_function.adam_fp16`` /
 ``adam_bf16``): fp32 master copy, moments and the 16-bit parameter are updated in a
-single pass over memory.  State layout per parameter (part of the checkpoint format):
+single pass over memory.  Parameters that lie back to back in one buffer (the flat
+per-block storage of ZeRO, whose gradients lie back to back too) get their state
+allocated back to back as well and are stepped by one launch over the whole run;
+small tensors elsewhere share launches; the rest take one launch per tensor.  State layout per parameter (part of the checkpoint format):
 ``step`` (int), ``exp_avg`` (fp16 for fp16 parameters, else fp32), ``exp_avg_sq``
 (fp32), ``_param_fp32`` (fp32 master, 16-bit parameters only).  For fp16 parameters
 the two moments are stored multiplied by the loss scale, which is why
@@ -12,6 +15,27 @@ import torch
 
 from . import _function as F
 from ._base import check_grad, remap_loaded_state, torch_adam_fp32, validate_hyper, wants_maximize
+
+
+def _follows(t, prev):
+    """True if contiguous tensor `t` starts where contiguous `prev` ends, inside the same storage."""
+    return (t.is_contiguous() and prev.is_contiguous() and t.dtype == prev.dtype
+            and t.data_ptr() == prev.data_ptr() + prev.numel() * prev.element_size()
+            and t.untyped_storage().data_ptr() == prev.untyped_storage().data_ptr())
+
+
+def _adjacent_runs(work):
+    """Splits 16-bit work items into maximal runs in which all five arrays of an item follow those of the
+    item before and step count and learning rate agree."""
+    runs = []
+    for item in work:
+        prev = runs[-1][-1] if runs else None
+        if (prev is not None and item[5] == prev[5] and item[6] == prev[6]
+                and all(_follows(a, b) for a, b in zip(item[:5], prev[:5]))):
+            runs[-1].append(item)
+        else:
+            runs.append([item])
+    return runs
 
 
 class AdamOptimizer(torch.optim.Optimizer):
@@ -28,6 +52,8 @@ class AdamOptimizer(torch.optim.Optimizer):
         # of their own: they stream at full rate either way, and slightly faster alone.
         self.batch_launches = True
         self.batch_below = 1 << 20
+        # Parameters, gradients and state that are adjacent in memory are stepped as one flat tensor.
+        self.merge_adjacent = True
 
     def _on_justify_scale(self, old_scale, new_scale):
         """fp16 moments are kept as moment * loss_scale (adam.py:46-55)."""
@@ -40,15 +66,38 @@ class AdamOptimizer(torch.optim.Optimizer):
                     state["exp_avg_sq"] *= ratio
 
     def _init_state(self, p):
-        moment_dtype = torch.float16 if p.dtype == torch.float16 else torch.float32
-        state = self.state[p]
-        state["step"] = 0
-        state["exp_avg"] = torch.zeros(p.size(), dtype=moment_dtype, device=p.device)
-        state["exp_avg_sq"] = torch.zeros(p.size(), dtype=torch.float32, device=p.device)
-        if p.dtype != torch.float32:
-            state["_param_fp32"] = torch.empty(p.size(), dtype=torch.float32, device=p.device)
-            state["_param_fp32"].copy_(p)
-        return state
+        self._init_states([p])
+        return self.state[p]
+
+    def _init_states(self, params):
+        """Creates the state of `params` (in order).  16-bit parameters that follow each other in memory
+        receive views into common flat buffers, so that the run can later be stepped by one launch."""
+        runs = []
+        for p in params:
+            last = runs[-1][-1] if runs else None
+            if (self.merge_adjacent and last is not None and p.dtype == last.dtype and p.dtype != torch.float32
+                    and _follows(p, last)):
+                runs[-1].append(p)
+            else:
+                runs.append([p])
+        for run in runs:
+            first = run[0]
+            total = sum(q.numel() for q in run)
+            moment_dtype = torch.float16 if first.dtype == torch.float16 else torch.float32
+            exp_avg = torch.zeros(total, dtype=moment_dtype, device=first.device)
+            exp_avg_sq = torch.zeros(total, dtype=torch.float32, device=first.device)
+            master = None if first.dtype == torch.float32 else torch.empty(total, dtype=torch.float32, device=first.device)
+            lo = 0
+            for q in run:
+                hi = lo + q.numel()
+                state = self.state[q]
+                state["step"] = 0
+                state["exp_avg"] = exp_avg[lo:hi].view(q.size())
+                state["exp_avg_sq"] = exp_avg_sq[lo:hi].view(q.size())
+                if master is not None:
+                    state["_param_fp32"] = master[lo:hi].view(q.size())
+                    state["_param_fp32"].copy_(q)
+                lo = hi
 
     @torch.no_grad()
     def step(self, closure=None, scale=1):
@@ -60,17 +109,15 @@ class AdamOptimizer(torch.optim.Optimizer):
 
         for group in self.param_groups:
             beta1, beta2 = group["betas"][0], group["betas"][1]
-            # 16-bit parameters of this group that can share launches: (dtype, step, lr) -> tensors
-            batches = {}
-            for p in group["params"]:
-                if p.grad is None or not p.requires_grad:
-                    continue
+            active = [p for p in group["params"] if p.grad is not None and p.requires_grad]
+            for p in active:
                 check_grad(p)
-                state = self.state[p]
-                if len(state) == 0:
-                    state = self._init_state(p)
-                grad = -p.grad if wants_maximize(group) else p.grad
+            self._init_states([p for p in active if len(self.state[p]) == 0])
 
+            half = []     # 16-bit work: (param_fp32, param, grad, exp_avg, exp_avg_sq, step, lr)
+            for p in active:
+                state = self.state[p]
+                grad = -p.grad if wants_maximize(group) else p.grad
                 if p.dtype == torch.float32:
                     # hold_steps is tested before the increment on this path (adam.py:137).
                     lr = 0.0 if state["step"] < self._hold_steps else group["lr"]
@@ -82,14 +129,21 @@ class AdamOptimizer(torch.optim.Optimizer):
                     # ... and after the increment on the fused path (adam.py:145,155).
                     state["step"] += 1
                     lr = 0.0 if state["step"] < self._hold_steps else group["lr"]
-                    if (self.batch_launches and p.numel() < self.batch_below
-                            and p.is_contiguous() and grad.is_contiguous()):
-                        batches.setdefault((p.dtype, state["step"], lr), []).append(
-                            (state["_param_fp32"], p, grad, state["exp_avg"], state["exp_avg_sq"]))
-                    else:
-                        fused = F.adam_fp16 if p.dtype == torch.float16 else F.adam_bf16
-                        fused(state["_param_fp32"], p, grad, state["exp_avg"], state["exp_avg_sq"],
-                              beta1, beta2, group["eps"], lr, scale, group["weight_decay"], state["step"])
+                    half.append((state["_param_fp32"], p, grad, state["exp_avg"], state["exp_avg_sq"], state["step"], lr))
+
+            # 16-bit parameters that can share launches: (dtype, step, lr) -> tensors
+            batches = {}
+            for run in _adjacent_runs(half) if self.merge_adjacent else [[w] for w in half]:
+                p32, p, grad, m, v, step, lr = run[0]
+                if len(run) > 1:
+                    total = sum(w[1].numel() for w in run)
+                    p32, p, grad, m, v = (t.as_strided((total,), (1,)) for t in (p32, p, grad, m, v))
+                elif (self.batch_launches and p.numel() < self.batch_below and p.is_contiguous()
+                        and grad.is_contiguous()):
+                    batches.setdefault((p.dtype, step, lr), []).append((p32, p, grad, m, v))
+                    continue
+                fused = F.adam_fp16 if p.dtype == torch.float16 else F.adam_bf16
+                fused(p32, p, grad, m, v, beta1, beta2, group["eps"], lr, scale, group["weight_decay"], step)
             for (_, step, lr), tensors in batches.items():
                 F.adam_multi(tensors, beta1, beta2, group["eps"], lr, scale, group["weight_decay"], step)
         return loss

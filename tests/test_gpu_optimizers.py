@@ -2,6 +2,7 @@
 tests/test_optim.py and the overflow handling of bmtrain/optim/optim_manager.py."""
 import copy
 
+import numpy as np
 import pytest
 import torch
 
@@ -117,6 +118,65 @@ def test_offload_in_pieces_equals_offload_in_one_call(dtype):
     assert abs(opt_c.get_avg_delta() - opt_w.get_avg_delta()) <= 1e-5 * abs(opt_w.get_avg_delta()) + 1e-9
     assert abs(opt_c.get_var_delta() - opt_w.get_var_delta()) <= 1e-4 * opt_w.get_var_delta()
     torch.testing.assert_close(cut._delta_info, whole._delta_info, rtol=1e-4, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_parameters_in_flat_storage_are_stepped_as_runs(dtype):
+    """Parameters that are views into one flat buffer (with gradients in another, as ZeRO blocks keep them)
+    get back-to-back state and one launch per run; results equal one launch per tensor bit for bit.  A
+    parameter without a gradient splits the run; a loaded state dict (separate tensors) ends the merging
+    without changing results."""
+    torch.manual_seed(5)
+    shapes = [(64, 4096), (4096,), (128, 128), (7,), (300001,), (33, 5)]
+    sizes = [int(np.prod(sh)) for sh in shapes]
+    total = sum(sizes)
+    flat_p = (torch.randn(total) * 0.02).to(dtype).cuda()
+    flat_g = torch.zeros(total, dtype=dtype, device="cuda")
+    merged, single = [], []
+    lo = 0
+    for sh, size in zip(shapes, sizes):
+        q = torch.nn.Parameter(flat_p[lo:lo + size].view(sh))
+        q.grad = flat_g[lo:lo + size].view(sh)
+        merged.append(q)
+        single.append(torch.nn.Parameter(flat_p[lo:lo + size].view(sh).clone()))
+        lo += size
+    opt_m = bmt.optim.AdamOptimizer(merged, lr=1e-3, weight_decay=0.01)
+    opt_s = bmt.optim.AdamOptimizer(single, lr=1e-3, weight_decay=0.01)
+    opt_s.merge_adjacent = False
+
+    def step(skip=None):
+        g = (torch.randn(total, device="cuda") * 1e-3 * 16).to(dtype)
+        flat_g.copy_(g)
+        lo = 0
+        for k, size in enumerate(sizes):
+            single[k].grad = None if k == skip else g[lo:lo + size].view(shapes[k]).clone()
+            if k == skip:
+                saved, merged[k].grad = merged[k].grad, None
+            lo += size
+        opt_m.step(scale=16); opt_s.step(scale=16)
+        if skip is not None:
+            merged[skip].grad = saved
+
+    def same():
+        for a, b in zip(merged, single):
+            assert torch.equal(a.detach().view(torch.int16), b.detach().view(torch.int16))
+            if len(opt_s.state[b]):
+                for key in ("_param_fp32", "exp_avg", "exp_avg_sq"):
+                    x, y = opt_m.state[a][key], opt_s.state[b][key]
+                    assert torch.equal(x.view(torch.int16 if x.element_size() == 2 else torch.int32),
+                                       y.view(torch.int16 if y.element_size() == 2 else torch.int32)), key
+                assert opt_m.state[a]["step"] == opt_s.state[b]["step"]
+
+    step(); step()
+    same()
+    storages = {opt_m.state[q]["exp_avg_sq"].untyped_storage().data_ptr() for q in merged}
+    assert len(storages) == 1                               # one flat state buffer for the whole run
+    step(skip=2)                                            # steps now differ inside the run: it splits
+    same()
+    step()
+    same()
+    opt_m.load_state_dict(copy.deepcopy(opt_m.state_dict()))   # separate tensors from here on
+    step(); same()
 
 
 def test_overflow_skips_the_step_and_halves_the_scale():
