@@ -50,6 +50,8 @@ def parse():
                     help="one transformer block (202,383,360 elements) and 2,048 rows: a quick functional run, "
                          "not the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the side measurements (other configurations, optimizer-level step); for profiler runs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed steps, run one plain device-to-device copy of the logits buffer "
                          "(rows * classes * 2 bytes read and written) so that rocprofv3 --pmc FETCH_SIZE / "
@@ -369,13 +371,14 @@ def main():
                            "frac": round(ce_gbps / HBM_PEAK_GBPS, 4), "bytes_per_row": ce_bytes_per_row(classes)},
         },
     }
-    tensor_list = None if args.small else {
+    side = not (args.small or args.no_other_workloads)
+    tensor_list = None if not side else {
         "adjacent_tensors_merged": tensor_list_step(torch, p16, grad, p32, mom, var, True),
         "one_launch_per_tensor": tensor_list_step(torch, p16, grad, p32, mom, var, False)}
     # free the device before the side measurements and the host baseline
     del p32, mom, var, grad, p16, logits, softmax
     torch.cuda.empty_cache()
-    if not args.small:
+    if side:
         result["other_workloads"] = other_workloads(torch, dev, LF, OF)
         result["other_workloads"]["adam_bf16_llama7b_291_tensors_via_optimizer_step"] = tensor_list
     if not args.no_cpu_baseline:
