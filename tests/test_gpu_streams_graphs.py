@@ -1,0 +1,96 @@
+"""The launchers are asynchronous on the caller's stream, allocate nothing and synchronise nothing, so a
+whole step can run on a side stream or be captured into a HIP graph and replayed."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from bmtrain_amd.loss import _function as LF
+from bmtrain_amd.optim import _function as OF
+from conftest import bits16, f32_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _state(n, seed, device="cuda"):
+    gen = torch.Generator().manual_seed(seed)
+    p = (torch.randn(n, generator=gen) * 0.02).to(device)
+    m = (torch.randn(n, generator=gen) * 1e-4).to(device)
+    v = (torch.randn(n, generator=gen) * 1e-6).abs().to(device)
+    g = (torch.randn(n, generator=gen) * 1e-3).bfloat16().to(device)
+    return p, torch.zeros(n, dtype=torch.bfloat16, device=device), g, m, v
+
+
+def _step(p, h, g, m, v, flag, x, t, soft, loss, go, step):
+    LF.has_inf_nan(g, flag)
+    OF.adam_bf16(p, h, g, m, v, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, step)
+    LF.cross_entropy_forward(x.size(0), x.size(1), x, t, soft, loss, -100)
+    LF.cross_entropy_backward_inplace(x.size(0), x.size(1), go, t, soft, -100)
+
+
+def _ce_inputs(rows, classes, seed):
+    gen = torch.Generator().manual_seed(seed)
+    x = (torch.randn(rows, classes, generator=gen) * 2).bfloat16().cuda()
+    t = torch.randint(0, classes, (rows,), generator=gen, dtype=torch.int32).cuda()
+    return x, t, torch.empty_like(x), torch.empty(rows, device="cuda"), torch.full((rows,), 1.0 / rows, device="cuda")
+
+
+@pytest.mark.parametrize("n", [100_003, (1 << 25) + 5])       # below and above the size where Adam tiles go by ticket
+def test_step_on_a_side_stream_equals_the_default_stream(n):
+    a, b = _state(n, 1), _state(n, 1)
+    ce_a, ce_b = _ce_inputs(64, 50257, 2), _ce_inputs(64, 50257, 2)
+    flag_a, flag_b = (torch.zeros(1, dtype=torch.uint8, device="cuda")[0] for _ in range(2))
+    _step(*a, flag_a, *ce_a, 3)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _step(*b, flag_b, *ce_b, 3)
+    side.synchronize()
+    torch.cuda.synchronize()
+    for x, y in zip(a + ce_a, b + ce_b):
+        assert torch.equal(x.view(torch.uint8), y.view(torch.uint8))
+    assert flag_a.item() == flag_b.item() == 0
+
+
+@pytest.mark.parametrize("n", [100_003, (1 << 25) + 5])
+def test_step_captured_in_a_graph_replays_like_eager(n):
+    """Four replays with eager work and synchronisation between them; every replay is compared with the same
+    step run eagerly on a twin state (and the first one with the oracle)."""
+    eager, graphed = _state(n, 7), _state(n, 7)
+    ce_e, ce_g = _ce_inputs(32, 32000, 8), _ce_inputs(32, 32000, 8)
+    flag_e, flag_g = (torch.zeros(1, dtype=torch.uint8, device="cuda")[0] for _ in range(2))
+    logits_static = ce_g[0]
+    before = [t.cpu().numpy().copy() if t.dtype == torch.float32 else bits16(t) for t in eager]
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                         # warm-up outside capture, on a scratch copy
+        scratch = tuple(t.clone() for t in graphed)
+        _step(*scratch, flag_g.clone(), *tuple(t.clone() for t in ce_g), 1)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _step(*graphed, flag_g, *ce_g, 1)               # the step number is baked into the captured arguments
+    # capture executes nothing: state is untouched
+    assert np.array_equal(f32_bits(graphed[0].cpu().numpy()), f32_bits(before[0]))
+
+    for replay in range(4):
+        new_logits = (torch.randn(32, 32000, device="cuda") * 2).bfloat16()     # eager work between replays
+        logits_static.copy_(new_logits); ce_e[0].copy_(new_logits)
+        graph.replay()
+        _step(*eager, flag_e, *ce_e, 1)
+        torch.cuda.synchronize()
+        for x, y in zip(eager + ce_e, graphed + ce_g):
+            assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), replay
+        if replay == 0:
+            p, h, g, m, v = before
+            bc1, bc2 = oracle.bias_corrections(0.9, 0.999, 1)
+            oracle.adam_gpu_bf16(p, h, g, m, v, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, bc1, bc2)
+            assert np.array_equal(f32_bits(graphed[0].cpu().numpy()), f32_bits(p))
+            assert np.array_equal(bits16(graphed[1]), h)
+    assert flag_g.item() == 0
+    graphed[2][17] = float("inf")                         # the captured scan sees the new gradient contents
+    graph.replay()
+    torch.cuda.synchronize()
+    assert flag_g.item() == 1
