@@ -95,3 +95,49 @@ def test_manager_scale_bookkeeping():
     loss = torch.tensor(2.0)
     assert m.scale_loss(loss).item() == 1024.0
     assert bmt.optim.OptimManager(loss_scale=8, grad_scale=4).scale_loss(loss).item() == 4.0
+
+
+def test_runs_of_adjacent_tensors():
+    """Which parameters the fused optimizer steps as one flat run: all five arrays back to back in one
+    storage each, same step count and learning rate."""
+    from bmtrain_amd.optim.adam import _adjacent_runs, _follows
+    flat = torch.zeros(100, dtype=torch.bfloat16)
+    a, b, c = flat[0:10], flat[10:40].view(5, 6), flat[41:50]
+    assert _follows(b, a) and not _follows(c, b) and not _follows(a, b)
+    assert not _follows(flat[10:40:2], a)                                  # not contiguous
+    assert not _follows(torch.zeros(30, dtype=torch.bfloat16), a)          # another storage
+    assert not _follows(flat.view(torch.float16)[10:40], a)                # another dtype
+
+    def item(lo, hi, step=3, lr=1e-3, bufs={}):
+        for name, dtype in (("p32", torch.float32), ("p", torch.bfloat16), ("g", torch.bfloat16), ("m", torch.float32),
+                            ("v", torch.float32)):
+            bufs.setdefault(name, torch.zeros(100, dtype=dtype))
+        return tuple(bufs[k][lo:hi] for k in ("p32", "p", "g", "m", "v")) + (step, lr)
+
+    work = [item(0, 10), item(10, 30), item(30, 31), item(32, 40), item(40, 50, step=4), item(50, 60, step=4, lr=0.0),
+            item(60, 70, step=4, lr=0.0)]
+    runs = _adjacent_runs(work)
+    assert [len(r) for r in runs] == [3, 1, 1, 2]
+    # one array out of line is enough to split
+    stray = list(item(70, 80, step=4, lr=0.0))
+    stray[2] = torch.zeros(10, dtype=torch.bfloat16)
+    assert [len(r) for r in _adjacent_runs(work + [tuple(stray)])] == [3, 1, 1, 2, 1]
+    assert _adjacent_runs([]) == []
+
+
+def test_state_of_adjacent_parameters_is_allocated_back_to_back():
+    flat = torch.zeros(64, dtype=torch.bfloat16)
+    params = [torch.nn.Parameter(flat[0:16].view(4, 4)), torch.nn.Parameter(flat[16:24]), torch.nn.Parameter(flat[30:40]),
+              torch.nn.Parameter(torch.zeros(5))]
+    opt = bmt.optim.AdamOptimizer(params, lr=1e-3)
+    opt._init_states(params)
+    s = [opt.state[p] for p in params]
+    assert s[0]["exp_avg"].shape == (4, 4) and s[0]["_param_fp32"].dtype == torch.float32
+    for key in ("exp_avg", "exp_avg_sq", "_param_fp32"):
+        assert s[1][key].data_ptr() == s[0][key].data_ptr() + 16 * 4
+        assert s[2][key].untyped_storage().data_ptr() != s[0][key].untyped_storage().data_ptr()
+    assert "_param_fp32" not in s[3] and s[3]["exp_avg"].dtype == torch.float32
+    opt.merge_adjacent = False
+    other = [torch.nn.Parameter(flat[40:48]), torch.nn.Parameter(flat[48:56])]
+    opt._init_states(other)
+    assert opt.state[other[1]]["exp_avg"].untyped_storage().data_ptr() != opt.state[other[0]]["exp_avg"].untyped_storage().data_ptr()
