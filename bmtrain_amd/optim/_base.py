@@ -10,6 +10,33 @@ import torch.optim._functional as _torch_functional
 SUPPORTED_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
 
 
+def follows(t, prev):
+    """True if contiguous tensor `t` starts where contiguous `prev` ends, inside the same storage."""
+    return (t.is_contiguous() and prev.is_contiguous() and t.dtype == prev.dtype
+            and t.data_ptr() == prev.data_ptr() + prev.numel() * prev.element_size()
+            and t.untyped_storage().data_ptr() == prev.untyped_storage().data_ptr())
+
+
+def flat_runs(tensors):
+    """Joins tensors that lie back to back in one storage (e.g. the gradients of a ZeRO block's flat
+    buffer) into flat 1-D views, in order; tensors that stand alone are passed through unchanged."""
+    out, run = [], []
+
+    def close():
+        if len(run) == 1:
+            out.append(run[0])
+        elif run:
+            out.append(run[0].as_strided((sum(t.numel() for t in run),), (1,)))
+        run.clear()
+
+    for t in tensors:
+        if run and not follows(t, run[-1]):
+            close()
+        run.append(t)
+    close()
+    return out
+
+
 def validate_hyper(lr, betas, eps, weight_decay):
     """ValueError texts follow torch.optim.Adam, as bmtrain/optim/adam.py:30-39 does."""
     if not 0.0 <= lr:

@@ -14,14 +14,7 @@ the two moments are stored multiplied by the loss scale, which is why
 import torch
 
 from . import _function as F
-from ._base import check_grad, remap_loaded_state, torch_adam_fp32, validate_hyper, wants_maximize
-
-
-def _follows(t, prev):
-    """True if contiguous tensor `t` starts where contiguous `prev` ends, inside the same storage."""
-    return (t.is_contiguous() and prev.is_contiguous() and t.dtype == prev.dtype
-            and t.data_ptr() == prev.data_ptr() + prev.numel() * prev.element_size()
-            and t.untyped_storage().data_ptr() == prev.untyped_storage().data_ptr())
+from ._base import check_grad, follows, remap_loaded_state, torch_adam_fp32, validate_hyper, wants_maximize
 
 
 def _adjacent_runs(work):
@@ -31,7 +24,7 @@ def _adjacent_runs(work):
     for item in work:
         prev = runs[-1][-1] if runs else None
         if (prev is not None and item[5] == prev[5] and item[6] == prev[6]
-                and all(_follows(a, b) for a, b in zip(item[:5], prev[:5]))):
+                and all(follows(a, b) for a, b in zip(item[:5], prev[:5]))):
             runs[-1].append(item)
         else:
             runs.append([item])
@@ -76,7 +69,7 @@ class AdamOptimizer(torch.optim.Optimizer):
         for p in params:
             last = runs[-1][-1] if runs else None
             if (self.merge_adjacent and last is not None and p.dtype == last.dtype and p.dtype != torch.float32
-                    and _follows(p, last)):
+                    and follows(p, last)):
                 runs[-1].append(p)
             else:
                 runs.append([p])

@@ -11,6 +11,7 @@ import torch
 
 from ..global_var import config
 from ..loss._function import has_inf_nan
+from ._base import flat_runs
 from ._function import grad_stats
 
 
@@ -18,10 +19,9 @@ def check_overflow(param_groups):
     """Raises OverflowError when any non-fp32 gradient holds an inf or NaN
     (optim_manager.py:9-21)."""
     flag = torch.zeros(1, dtype=torch.uint8, device="cuda")[0]
-    for group in param_groups:
-        for p in group["params"]:
-            if p.grad is not None and p.dtype != torch.float:
-                has_inf_nan(p.grad, flag)
+    grads = [p.grad for group in param_groups for p in group["params"] if p.grad is not None and p.dtype != torch.float]
+    for g in flat_runs(grads):      # gradients that lie back to back are scanned by one launch
+        has_inf_nan(g, flag)
     if flag > 0:
         raise OverflowError("Gradient overflow")
 
@@ -136,7 +136,7 @@ class OptimManager:
                 # 16-bit gradients: one read of each tensor instead of an fp32 copy plus a norm
                 sumsq = torch.zeros(1, dtype=torch.float64, device=device)
                 flag = torch.zeros(1, dtype=torch.uint8, device=device)
-                for g in fused:
+                for g in flat_runs(fused):
                     grad_stats(g, sumsq, flag)
                 acc += sumsq.float()
             fused_ids = {id(g) for g in fused}

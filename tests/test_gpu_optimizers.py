@@ -179,6 +179,35 @@ def test_parameters_in_flat_storage_are_stepped_as_runs(dtype):
     step(); same()
 
 
+def test_overflow_check_and_grad_norm_over_flat_gradient_storage():
+    """Gradients that are views into one buffer are scanned as one run: same verdicts and norm as tensor by tensor."""
+    from bmtrain_amd.optim.optim_manager import check_overflow
+    torch.manual_seed(6)
+    sizes = [4096, 7, 100003, 64 * 64]
+    flat_g = (torch.randn(sum(sizes), device="cuda") * 64).bfloat16()
+    params, lo = [], 0
+    for size in sizes:
+        q = torch.nn.Parameter(torch.zeros(size, dtype=torch.bfloat16, device="cuda"))
+        q.grad = flat_g[lo:lo + size]
+        params.append(q)
+        lo += size
+    lone = torch.nn.Parameter(torch.zeros(33, dtype=torch.float16, device="cuda"))
+    lone.grad = torch.ones(33, dtype=torch.float16, device="cuda")
+    groups = [{"params": params + [lone]}]
+    check_overflow(groups)                                   # finite: no exception
+    manager = bmt.optim.OptimManager(loss_scale=64)
+    want = torch.cat([flat_g.float(), lone.grad.float()]).norm() / 64
+    got = manager.clip_grad_norm(groups, max_norm=1e9)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=0)
+    flat_g[4096 + 7 + 50000] = float("nan")                  # inside the third tensor of the run
+    with pytest.raises(OverflowError):
+        check_overflow(groups)
+    flat_g[4096 + 7 + 50000] = 0
+    lone.grad[32] = float("inf")
+    with pytest.raises(OverflowError):
+        check_overflow(groups)
+
+
 def test_overflow_skips_the_step_and_halves_the_scale():
     torch.manual_seed(2)
     p = torch.nn.Parameter(torch.randn(1000, device="cuda").half())

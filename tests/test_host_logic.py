@@ -100,13 +100,17 @@ def test_manager_scale_bookkeeping():
 def test_runs_of_adjacent_tensors():
     """Which parameters the fused optimizer steps as one flat run: all five arrays back to back in one
     storage each, same step count and learning rate."""
-    from bmtrain_amd.optim.adam import _adjacent_runs, _follows
+    from bmtrain_amd.optim.adam import _adjacent_runs
+    from bmtrain_amd.optim._base import flat_runs, follows as _follows
     flat = torch.zeros(100, dtype=torch.bfloat16)
     a, b, c = flat[0:10], flat[10:40].view(5, 6), flat[41:50]
     assert _follows(b, a) and not _follows(c, b) and not _follows(a, b)
     assert not _follows(flat[10:40:2], a)                                  # not contiguous
     assert not _follows(torch.zeros(30, dtype=torch.bfloat16), a)          # another storage
     assert not _follows(flat.view(torch.float16)[10:40], a)                # another dtype
+    joined = flat_runs([a, b, c, torch.zeros(3, dtype=torch.bfloat16), flat[50:60], flat[60:100]])
+    assert [t.numel() for t in joined] == [40, 9, 3, 50] and joined[0].data_ptr() == flat.data_ptr()
+    assert joined[1] is c and flat_runs([]) == []
 
     def item(lo, hi, step=3, lr=1e-3, bufs={}):
         for name, dtype in (("p32", torch.float32), ("p", torch.bfloat16), ("g", torch.bfloat16), ("m", torch.float32),
