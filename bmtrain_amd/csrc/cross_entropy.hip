@@ -10,10 +10,9 @@
 // row and moves it as 16-byte vectors:
 //   * up to 32,768 elements the row is read once into registers; maximum, exponentials (kept in
 //     fp32 registers), sum and quotient all work on registers (ce_forward_row_kernel);
-//   * up to 131,072 elements the row is streamed once while a per-lane running maximum / sum is
-//     kept; 4 vectors per lane stay in registers and up to 4 in LDS, the remainder is fetched a
-//     second time for the output sweep (ce_forward_retain_kernel);
-//   * longer rows are streamed twice (ce_forward_stream_kernel).
+//   * longer rows are streamed once while a per-lane running maximum / sum is kept; 4 vectors
+//     per lane stay in registers and up to 4 in LDS (65,536 elements), the remainder is fetched a
+//     second time for the output sweep (ce_forward_retain_kernel).
 // Reductions are a wave64 butterfly followed by one LDS slot per wave.  Rows may have any length
 // and start at any 2-byte offset: each row is split into a head of fewer than 8 elements, whole
 // 16-byte vectors and a tail (RowSpan).  Only when logits and softmax sit at different offsets
@@ -210,94 +209,22 @@ __device__ __forceinline__ u32x4 vec_softmax(const u32x4 &w, float M, const RowS
     return o;
 }
 
-// ---- forward, long rows: two sweeps, the second one served by the caches ------------
-// Sweep 1 reads the row from HBM and keeps, per lane, a running maximum and the sum of
-// exponentials relative to it (rescaled when the maximum grows); nothing is stored on chip,
-// so several workgroups per CU overlap their memory and ALU phases.  Sweep 2 reads the row
-// again — it was just fetched with the default cache policy, so L2 / Infinity Cache still hold
-// it — and writes the quotient.  THREADS lanes per row, UNROLL vectors per lane per step.
-template <typename T, int THREADS, int UNROLL>
-__global__ __launch_bounds__(THREADS) void ce_forward_stream_kernel(
-    int32_t n, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
-    uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
-    __shared__ float slots[2][THREADS / kWave];
-    const int64_t row = blockIdx.x;
-    const RowSpan sp = row_span(x, row, n);
-    const int32_t nvec = sp.nvec;
-    const u32x4 *xr = (const u32x4 *)(sp.row + sp.head);
-    uint16_t *srow = softmax + row * n;
-    u32x4 *sr = (u32x4 *)(srow + sp.head);
-    const int tid = threadIdx.x;
-    const uint32_t pad = neg_inf2<T>();
-    const u32x4 pad4 = {pad, pad, pad, pad};
-
-    float m = -1e6f;          // running maximum of this lane, never below the reference's clamp
-    float s = 0.f;            // sum of 2^64 * e^(x - m) over this lane's elements so far
-    for (int j0 = 0; j0 < nvec; j0 += THREADS * UNROLL) {
-        u32x4 w[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
-            const int j = j0 + u * THREADS + tid;
-            w[u] = j < nvec ? xr[j] : pad4;
-        }
-        float vm = -INFINITY;
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) vec_max<T>(w[u], vm);
-        if (vm > m) {   // rare after the first steps
-            s *= __builtin_amdgcn_exp2f((m - vm) * kLog2e);
-            m = vm;
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) vec_sumexp<T>(w[u], m, s);
-    }
-    if (tid < sp.nedge) {
-        const float edge = T::to_f32(sp.row[sp.edge_index(tid)]);
-        if (edge > m) {
-            s *= __builtin_amdgcn_exp2f((m - edge) * kLog2e);
-            m = edge;
-        }
-        s += exp_biased(edge, m);
-    }
-    const float M = block_allreduce<true>(m, slots[0]);
-    s *= __builtin_amdgcn_exp2f((m - M) * kLog2e);
-    const RowSum rs = make_row_sum(block_allreduce<false>(s, slots[1]));
-    if (tid < sp.nedge) {
-        const int32_t i = sp.edge_index(tid);
-        srow[i] = T::from_f32(quotient(exp_biased(T::to_f32(sp.row[i]), M), rs));
-    }
-
-    for (int j0 = 0; j0 < nvec; j0 += THREADS * UNROLL) {
-        u32x4 w[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
-            const int j = j0 + u * THREADS + tid;
-            w[u] = j < nvec ? xr[j] : pad4;
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
-            const int j = j0 + u * THREADS + tid;
-            if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(w[u], M, rs), sr + j);
-        }
-    }
-    if (tid == 0) out[row] = row_loss<T>(sp.row, n, target[row], ignore_index, M, rs.S);
-}
-
 // ---- forward, long rows: stream once, keep most of the row on chip ---------------------
 // 1024 lanes per row, two workgroups per CU (<= 64 VGPRs, <= 64 KiB LDS each).  Sweep 1 streams
-// the row from HBM in CHUNKS vectors per lane while each lane keeps a running maximum and the sum
+// the row from HBM in `chunks` vectors per lane while each lane keeps a running maximum and the sum
 // of exponentials relative to it (rescaled when the maximum grows).  The first RK vectors of a
 // lane stay in registers and the next LK in LDS; the remaining ones are dropped.  Sweep 2 walks the
 // row backwards: the dropped vectors — the most recently fetched, so the likeliest to sit in L2
 // still — are loaded again, then the LDS and register parts follow without memory traffic.
 // Fine-grained load/compute interleaving in both sweeps lets the 32 waves of a CU hide each
 // other's latencies, which a whole-row-resident scheme with one or two workgroups per CU cannot.
-template <typename T, int CHUNKS, int RK, int LK>
+template <typename T, int RK, int LK>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void ce_forward_retain_kernel(
     int32_t n, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
-    uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
+    uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index, int32_t chunks) {
     constexpr int THREADS = 1024;
     constexpr int GROUP = 2;
-    static_assert(CHUNKS % GROUP == 0 && RK % GROUP == 0 && LK % GROUP == 0, "chunk counts must be even");
+    static_assert(RK % GROUP == 0 && LK % GROUP == 0, "chunk counts must be even");   // and so is `chunks`
     extern __shared__ u32x4 staged[];  // LK * 1024 vectors
     __shared__ float slots[2][THREADS / kWave];
     const int64_t row = blockIdx.x;
@@ -355,7 +282,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
     }
     // dropped part: default cache policy, meant to be found in L2 again
 #pragma unroll 1
-    for (int c0 = RK + LK; c0 < CHUNKS; c0 += GROUP) {
+    for (int c0 = RK + LK; c0 < chunks; c0 += GROUP) {
         u32x4 v[GROUP];
 #pragma unroll
         for (int g = 0; g < GROUP; g++) {
@@ -382,7 +309,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
 
     // dropped part, last fetched first
 #pragma unroll 1
-    for (int c0 = CHUNKS - GROUP; c0 >= RK + LK; c0 -= GROUP) {
+    for (int c0 = chunks - GROUP; c0 >= RK + LK; c0 -= GROUP) {
         u32x4 v[GROUP];
 #pragma unroll
         for (int g = GROUP - 1; g >= 0; g--) {
@@ -572,20 +499,16 @@ static int flat_grid(int64_t work_items, int threads_times_unroll) {
                        (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,     \
                        ignore_index)
 
-#define BMT_CE_STREAM(THREADS, UNROLL)                                                                             \
-    hipLaunchKernelGGL((ce_forward_stream_kernel<T, THREADS, UNROLL>), dim3((unsigned)m), dim3(THREADS), 0, s, n,       \
-                       (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,     \
-                       ignore_index)
-
 #define BMT_CE_RETAIN(CHUNKS, RK, LK)                                                                              \
     do {                                                                                                           \
-        auto kern = ce_forward_retain_kernel<T, CHUNKS, RK, LK>;                                                   \
+        auto kern = ce_forward_retain_kernel<T, RK, LK>;                                                           \
         const size_t lds = (size_t)(LK) * 1024 * sizeof(u32x4);                                                    \
         static const hipError_t attr = hipFuncSetAttribute((const void *)kern,                                     \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);  \
         if (attr != hipSuccess) return fail((int)attr, who, attr);                                                 \
         hipLaunchKernelGGL(kern, dim3((unsigned)m), dim3(1024), lds, s, n, (const uint16_t *)input,                \
-                           (const int32_t *)target, (uint16_t *)softmax, (float *)output, ignore_index);           \
+                           (const int32_t *)target, (uint16_t *)softmax, (float *)output, ignore_index,            \
+                           (int32_t)(CHUNKS));                                                                     \
     } while (0)
 
 template <typename T>
@@ -612,13 +535,8 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
         else if (nvec <= 4096) BMT_CE_ROW(1024, 4);
         // up to 65,536 elements: 4 vectors per lane in registers, the rest in LDS, two workgroups per CU
         else if (nvec <= 6144) BMT_CE_RETAIN(6, 2, 4);
-        else if (nvec <= 8192) BMT_CE_RETAIN(8, 4, 4);
-        // up to 131,072 elements: 8 vectors per lane kept, the rest fetched twice
-        else if (nvec <= 10240) BMT_CE_RETAIN(10, 4, 4);
-        else if (nvec <= 12288) BMT_CE_RETAIN(12, 4, 4);
-        else if (nvec <= 14336) BMT_CE_RETAIN(14, 4, 4);
-        else if (nvec <= 16384) BMT_CE_RETAIN(16, 4, 4);
-        else BMT_CE_STREAM(1024, 2);
+        // longer rows: 8 vectors per lane kept, the rest fetched twice
+        else BMT_CE_RETAIN(2 * ((nvec + 2047) / 2048), 4, 4);
     } else {
         hipLaunchKernelGGL((ce_forward_sweep_kernel<T>), dim3((unsigned)m), dim3(kSweepThreads), 0, s, n,
                            (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,
