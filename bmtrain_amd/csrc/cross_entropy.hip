@@ -21,6 +21,7 @@
 //
 // Backward (reference kernels :46-60, :104-121), element-wise and in place on the
 // stored softmax: x[r, i] = to16((x[r, i] - (i == target[r])) * grad_output[r]).
+#include <atomic>
 #include "bmt_device.h"
 #include "bmt_host.h"
 #include "../../include/bmt_hip.h"
@@ -503,9 +504,15 @@ static int flat_grid(int64_t work_items, int threads_times_unroll) {
     do {                                                                                                           \
         auto kern = ce_forward_retain_kernel<T, RK, LK>;                                                           \
         const size_t lds = (size_t)(LK) * 1024 * sizeof(u32x4);                                                    \
-        static const hipError_t attr = hipFuncSetAttribute((const void *)kern,                                     \
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);  \
-        if (attr != hipSuccess) return fail((int)attr, who, attr);                                                 \
+        static std::atomic<uint64_t> allowed{0};   /* devices on which this kernel may use `lds` bytes */         \
+        int dev = 0;                                                                                               \
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 63;                                    \
+        if (dev == 63 || !((allowed.load(std::memory_order_relaxed) >> dev) & 1u)) {                               \
+            const hipError_t attr = hipFuncSetAttribute((const void *)kern,                                        \
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);     \
+            if (attr != hipSuccess) return fail((int)attr, who, attr);                                             \
+            allowed.fetch_or((uint64_t)1 << dev, std::memory_order_relaxed);                                       \
+        }                                                                                                          \
         hipLaunchKernelGGL(kern, dim3((unsigned)m), dim3(1024), lds, s, n, (const uint16_t *)input,                \
                            (const int32_t *)target, (uint16_t *)softmax, (float *)output, ignore_index,            \
                            (int32_t)(CHUNKS));                                                                     \
