@@ -133,9 +133,10 @@ def cpu_baseline():
 
 
 def other_workloads(torch, dev, LF, OF, iters=20):
-    """The two single-kernel configurations the targets are also stated on (not the headline line):
-    one transformer block's flat Adam step (202,383,360 elements, bf16, t = 100) and the fp16 language-model
-    head cross-entropy (16,384 rows x 32,000 classes, 10 % ignored)."""
+    """The other configurations the targets are stated on (not the headline line): one transformer block's
+    flat Adam step (202,383,360 elements, bf16, t = 100; also fp16 and the gradient statistics pass over the
+    same gradients), the fp16 overflow scan over 2^30 elements, and the fp16 language-model head
+    cross-entropy (16,384 rows x 32,000 classes, 10 % ignored)."""
     def timed(fn):
         for _ in range(3):
             fn()
@@ -172,6 +173,16 @@ def other_workloads(torch, dev, LF, OF, iters=20):
     gbps = 2 * n / (ms * 1e-3) / 1e9
     out["grad_stats_bf16_202M"] = {"ms": round(ms, 4), "achieved_GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
     del p16, grad, p32, mom, var, h16, g16, m16
+    torch.cuda.empty_cache()
+
+    n16 = 1 << 30
+    g = torch.empty(n16, dtype=torch.float16, device=dev)
+    fill_normal_(g, 1e-3, gen)
+    flag = torch.zeros(1, dtype=torch.uint8, device=dev)[0]
+    ms = timed(lambda: LF.has_inf_nan(g, flag))
+    gbps = SCAN_BYTES * n16 / (ms * 1e-3) / 1e9
+    out["has_inf_nan_fp16_2^30"] = {"ms": round(ms, 4), "achieved_GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+    del g
     torch.cuda.empty_cache()
 
     gen = torch.Generator(device=dev).manual_seed(3)
