@@ -7,10 +7,10 @@
 // that makes an all-ones field carry into bit 15 of its half; no other field value
 // reaches bit 15, and the mask keeps the low half's carry out of the high half:
 //     hit |= ((w & EXP_MASK2) + EXP_CARRY2) & 0x80008000
-// Each lane ORs its dwords, the wave votes with one ballot, the waves of a
-// workgroup meet in one LDS word, and one lane per workgroup that saw a hit issues
-// a single relaxed atomic byte store out[0] = 1.  When nothing is found the
-// kernel writes nothing, which keeps the flag sticky across calls.
+// Each lane ORs its dwords, the wave votes with one ballot, and one lane of a wave
+// that saw a hit issues a relaxed atomic byte store out[0] = 1 (after a look at the
+// flag: once it is up nobody stores again).  When nothing is found the kernel writes
+// nothing, which keeps the flag sticky across calls.
 #include "bmt_device.h"
 #include "bmt_host.h"
 #include "../../include/bmt_hip.h"
@@ -18,9 +18,11 @@
 namespace bmt {
 
 // One workgroup scans one tile of kScanThreads * UNROLL 16-byte vectors and exits (short
-// workgroups stream faster here than a resident grid that loops).
+// workgroups stream faster here than a resident grid that loops; one vector per lane and no
+// workgroup-level meeting point measured 94 % of HBM peak, two vectors with an LDS word and two
+// barriers 89 %).
 constexpr int kScanThreads = 1024;
-constexpr int kScanUnroll = 2;
+constexpr int kScanUnroll = 1;
 // The statistics kernel ends in a workgroup-wide sum; a four times larger tile (128 KiB) spreads
 // that cost and keeps eight loads per lane in flight.
 constexpr int kStatsUnroll = 8;
@@ -55,13 +57,10 @@ __global__ __launch_bounds__(kScanThreads) void has_inf_nan_kernel(
             hit |= exp_all_ones2<T>((uint32_t)g[i]);
         }
     }
-    __shared__ uint32_t any_wave;
-    if (threadIdx.x == 0) any_wave = 0;
-    __syncthreads();
-    const bool wave_hit = __builtin_amdgcn_ballot_w64(hit != 0) != 0;
-    if (wave_hit && (threadIdx.x & (kWave - 1)) == 0) any_wave = 1;
-    __syncthreads();
-    if (threadIdx.x == 0 && any_wave)
+    // Each wave votes on its own (no LDS, no barrier); a wave that saw a hit raises the flag unless
+    // it is up already, so a buffer full of NaNs costs a few stores, not one per wave.
+    if (__builtin_amdgcn_ballot_w64(hit != 0) != 0 && (threadIdx.x & (kWave - 1)) == 0 &&
+        __hip_atomic_load(out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
         __hip_atomic_store(out, (uint8_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
