@@ -6,8 +6,9 @@
 //   M = max(max_i x_i, -1e6);  S = sum_i expf(x_i - M) + 1e-10
 //   softmax[r, i] = to16(expf(x_i - M) / S)
 //   out[r] = target[r] != ignore ? (-x[target[r]] + M) + logf(S) : 0
-// The reference walks each row three times from global memory.  Here one workgroup owns a
-// row and moves it as 16-byte vectors:
+// The reference walks each row three times from global memory.  Here rows move as 16-byte
+// vectors; rows of up to 512 elements share a wave (ce_forward_small_kernel), longer ones get a
+// workgroup each:
 //   * up to 32,768 elements the row is read once into registers; maximum, exponentials (kept in
 //     fp32 registers), sum and quotient all work on registers (ce_forward_row_kernel);
 //   * longer rows are streamed once while a per-lane running maximum / sum is kept; 4 vectors
@@ -208,6 +209,92 @@ __device__ __forceinline__ u32x4 vec_softmax(const u32x4 &w, float M, const RowS
     for (int k = 0; k < 4; k++)
         o[k] = pack2<T>(quotient(exp_biased(lo_f32<T>(w[k]), M), rs), quotient(exp_biased(hi_f32<T>(w[k]), M), rs));
     return o;
+}
+
+// ---- forward, short rows ---------------------------------------------------------------
+// Rows of up to 64 vectors.  LANES (8..64) adjacent lanes own one row, one vector per lane, so a
+// wave holds 64 / LANES rows side by side; it works on R such sets at once, with all loads issued
+// first (a single 1 KiB row per wave in flight would leave HBM idle).  Reductions are butterflies
+// inside the lane group; no LDS, no barriers.  256 lanes per workgroup.
+constexpr int kSmallThreads = 256;
+template <int LANES, bool IsMax>
+__device__ __forceinline__ float group_allreduce(float v) {
+#pragma unroll
+    for (int off = LANES / 2; off > 0; off >>= 1) {
+        const float o = __shfl_xor(v, off, kWave);
+        v = IsMax ? fmaxf(v, o) : v + o;
+    }
+    return v;
+}
+template <typename T, int LANES, int R>
+__global__ __launch_bounds__(kSmallThreads) void ce_forward_small_kernel(
+    int32_t m, int32_t n, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
+    uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
+    constexpr int GROUPS = kWave / LANES;                          // rows side by side in a wave
+    const int lane = threadIdx.x & (kWave - 1);
+    const int sub = lane & (LANES - 1);                            // lane inside its row
+    const int64_t wave_id = (int64_t)blockIdx.x * (kSmallThreads / kWave) + threadIdx.x / kWave;
+    const int64_t row0 = wave_id * (R * GROUPS) + lane / LANES;     // set r covers rows row0 + r * GROUPS
+
+    RowSpan sp[R];
+    u32x4 w[R];
+    bool live[R];                                                  // this lane holds a vector of its row
+    const uint32_t pad = neg_inf2<T>();
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int64_t row = row0 + (int64_t)r * GROUPS;
+        const bool row_ok = row < m;
+        sp[r] = row_span(x, row_ok ? row : 0, n);
+        if (!row_ok) { sp[r].nvec = 0; sp[r].nedge = 0; }
+        live[r] = sub < sp[r].nvec;
+        if (live[r]) w[r] = __builtin_nontemporal_load((const u32x4 *)(sp[r].row + sp[r].head) + sub);
+        else { w[r].x = pad; w[r].y = pad; w[r].z = pad; w[r].w = pad; }
+    }
+    float M[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float mx = -INFINITY;
+        if (live[r]) vec_max<T>(w[r], mx);
+        for (int e = sub; e < sp[r].nedge; e += LANES) mx = fmaxf(T::to_f32(sp[r].row[sp[r].edge_index(e)]), mx);
+        M[r] = fmaxf(group_allreduce<LANES, true>(mx), -1e6f);
+    }
+    float ex[R][8];
+    RowSum rs[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float sum = 0.f;
+        if (live[r]) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                ex[r][2 * k] = exp_biased(lo_f32<T>(w[r][k]), M[r]);
+                ex[r][2 * k + 1] = exp_biased(hi_f32<T>(w[r][k]), M[r]);
+                sum += ex[r][2 * k];
+                sum += ex[r][2 * k + 1];
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) ex[r][k] = 0.f;
+        }
+        for (int e = sub; e < sp[r].nedge; e += LANES) sum += exp_biased(T::to_f32(sp[r].row[sp[r].edge_index(e)]), M[r]);
+        rs[r] = make_row_sum(group_allreduce<LANES, false>(sum));
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int64_t row = row0 + (int64_t)r * GROUPS;
+        if (row >= m) continue;
+        uint16_t *srow = softmax + row * n;
+        if (live[r]) {
+            u32x4 o;
+#pragma unroll
+            for (int k = 0; k < 4; k++) o[k] = pack2<T>(quotient(ex[r][2 * k], rs[r]), quotient(ex[r][2 * k + 1], rs[r]));
+            __builtin_nontemporal_store(o, (u32x4 *)(srow + sp[r].head) + sub);
+        }
+        for (int e = sub; e < sp[r].nedge; e += LANES) {
+            const int32_t i = sp[r].edge_index(e);
+            srow[i] = T::from_f32(quotient(exp_biased(T::to_f32(sp[r].row[i]), M[r]), rs[r]));
+        }
+        if (sub == 0) out[row] = row_loss<T>(sp[r].row, n, target[row], ignore_index, M[r], rs[r].S);
+    }
 }
 
 // ---- forward, long rows: stream once, keep most of the row on chip ---------------------
@@ -500,6 +587,15 @@ static int flat_grid(int64_t work_items, int threads_times_unroll) {
                        (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,     \
                        ignore_index)
 
+#define BMT_CE_SMALL(LANES)                                                                                       \
+    do {                                                                                                           \
+        constexpr int R = 2;                                                                                       \
+        const int64_t rows_per_group = (int64_t)(kSmallThreads / kWave) * R * (kWave / (LANES));                   \
+        hipLaunchKernelGGL((ce_forward_small_kernel<T, LANES, R>), dim3((unsigned)((m + rows_per_group - 1) / rows_per_group)), \
+                           dim3(kSmallThreads), 0, s, m, n, (const uint16_t *)input, (const int32_t *)target,      \
+                           (uint16_t *)softmax, (float *)output, ignore_index);                                    \
+    } while (0)
+
 #define BMT_CE_RETAIN(CHUNKS, RK, LK)                                                                              \
     do {                                                                                                           \
         auto kern = ce_forward_retain_kernel<T, RK, LK>;                                                           \
@@ -529,7 +625,11 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
     const int32_t nvec = n / 8;   // the most vectors a row can have
     if (same_vector_phase(input, softmax)) {
         // rows up to 32,768 elements live in the registers of their workgroup
-        if (nvec <= 64) BMT_CE_ROW(64, 1);
+        // short rows: several rows per wave
+        if (nvec <= 8) BMT_CE_SMALL(8);
+        else if (nvec <= 16) BMT_CE_SMALL(16);
+        else if (nvec <= 32) BMT_CE_SMALL(32);
+        else if (nvec <= 64) BMT_CE_SMALL(64);
         else if (nvec <= 128) BMT_CE_ROW(64, 2);
         else if (nvec <= 192) BMT_CE_ROW(64, 3);
         else if (nvec <= 256) BMT_CE_ROW(64, 4);
