@@ -459,7 +459,12 @@ constexpr int kFlatScalarThreads = 256;
 template <typename T, int OP>
 __device__ __forceinline__ float flat_elem(float s, bool is_target, float a, float b) {
     if (OP == 0) return is_target ? (s - 1.f) * a : s * a;  // a = grad_output[r]
-    return expf(s - a) / b;                                 // a = max, b = sum
+    return exp_biased(s, a) * b;                            // a = max, b = 2^-64 / sum
+}
+// Second per-row scalar of the flat kernels: nothing for the backward, 2^-64 / sum for the softmax.
+template <int OP>
+__device__ __forceinline__ float flat_row_b(const float *row_b, int64_t row) {
+    return OP == 1 ? kTwoPowMinusBias / row_b[row] : 0.f;
 }
 
 // One workgroup transforms one tile of kFlatThreads * kFlatUnroll vectors and exits.  The array is
@@ -493,7 +498,7 @@ __global__ __launch_bounds__(kFlatThreads) void ce_flat_vec_kernel(
         const int64_t row = row0 + dr;
         const int32_t col = (int32_t)(off - dr * (uint32_t)n);
         const float a = row_a[row];
-        const float b = OP == 1 ? row_b[row] : 0.f;
+        const float b = flat_row_b<OP>(row_b, row);
         const int32_t tk = OP == 0 ? target[row] - col : -1;  // position of the target inside this vector
         u32x4 o;
         if (!RAGGED || col + 8 <= n) {
@@ -506,7 +511,7 @@ __global__ __launch_bounds__(kFlatThreads) void ce_flat_vec_kernel(
         } else {   // elements from position `split` on belong to the next row
             const int32_t split = n - col;
             const float a1 = row_a[row + 1];
-            const float b1 = OP == 1 ? row_b[row + 1] : 0.f;
+            const float b1 = flat_row_b<OP>(row_b, row + 1);
             const int32_t tk1 = OP == 0 ? target[row + 1] + split : -1;
 #pragma unroll
             for (int k = 0; k < 4; k++) {
@@ -528,7 +533,7 @@ __global__ __launch_bounds__(kFlatThreads) void ce_flat_vec_kernel(
             const int64_t row = i / n;
             const int32_t col = (int32_t)(i - row * n);
             const bool is_t = OP == 0 ? (target[row] == col) : false;
-            x[i] = T::from_f32(flat_elem<T, OP>(T::to_f32(x[i]), is_t, row_a[row], OP == 1 ? row_b[row] : 0.f));
+            x[i] = T::from_f32(flat_elem<T, OP>(T::to_f32(x[i]), is_t, row_a[row], flat_row_b<OP>(row_b, row)));
         }
     }
 }
@@ -542,31 +547,37 @@ __global__ __launch_bounds__(kFlatScalarThreads) void ce_flat_scalar_kernel(
         const int64_t row = g / n;
         const int32_t col = (int32_t)(g - row * n);
         const float a = row_a[row];
-        const float b = OP == 1 ? row_b[row] : 0.f;
+        const float b = flat_row_b<OP>(row_b, row);
         const bool is_t = OP == 0 ? (target[row] == col) : false;
         x[g] = T::from_f32(flat_elem<T, OP>(T::to_f32(x[g]), is_t, a, b));
     }
 }
 
 // ---- row sum of exponentials given the row maximum ---------------------------------
-template <typename T>
-__global__ __launch_bounds__(kSweepThreads) void sumexp_kernel(int32_t n, const uint16_t *__restrict__ x,
-                                                               const float *__restrict__ row_max,
-                                                               float *__restrict__ row_sum) {
-    __shared__ float slots[kSweepThreads / kWave];
+// One workgroup of THREADS lanes per row, two vectors per lane in flight.  The exponentials are the
+// biased ones of the forward kernels; the factor 2^64 is taken out of the sum at the end.
+template <typename T, int THREADS>
+__global__ __launch_bounds__(THREADS) void sumexp_kernel(int32_t n, const uint16_t *__restrict__ x,
+                                                         const float *__restrict__ row_max,
+                                                         float *__restrict__ row_sum) {
+    __shared__ float slots[THREADS / kWave];
     const int64_t row = blockIdx.x;
     const RowSpan sp = row_span(x, row, n);
     const u32x4 *xr = (const u32x4 *)(sp.row + sp.head);
     const float M = row_max[row];
+    const uint32_t pad = neg_inf2<T>();
+    const u32x4 pad4 = {pad, pad, pad, pad};
     float sum = 0.f;
-    for (int j = threadIdx.x; j < sp.nvec; j += kSweepThreads) {
-        const u32x4 w = __builtin_nontemporal_load(xr + j);
-#pragma unroll
-        for (int k = 0; k < 4; k++) { sum += expf(lo_f32<T>(w[k]) - M); sum += expf(hi_f32<T>(w[k]) - M); }
+    for (int j0 = 0; j0 < sp.nvec; j0 += 2 * THREADS) {
+        const int ja = j0 + threadIdx.x, jb = ja + THREADS;
+        const u32x4 wa = ja < sp.nvec ? __builtin_nontemporal_load(xr + ja) : pad4;
+        const u32x4 wb = jb < sp.nvec ? __builtin_nontemporal_load(xr + jb) : pad4;
+        vec_sumexp<T>(wa, M, sum);
+        vec_sumexp<T>(wb, M, sum);
     }
-    if ((int)threadIdx.x < sp.nedge) sum += expf(T::to_f32(sp.row[sp.edge_index(threadIdx.x)]) - M);
+    if ((int)threadIdx.x < sp.nedge) sum += exp_biased(T::to_f32(sp.row[sp.edge_index(threadIdx.x)]), M);
     sum = block_allreduce<false>(sum, slots);
-    if (threadIdx.x == 0) row_sum[row] = sum;
+    if (threadIdx.x == 0) row_sum[row] = sum * kTwoPowMinusBias;
 }
 
 // ---- host side ------------------------------------------------------------------
@@ -687,8 +698,12 @@ static int sumexp(int32_t m, int32_t n, const void *logits, const void *row_max,
     if (!logits || !row_max || !row_sum) return fail(-1, "fused_sumexp launcher: null pointer");
     hipStream_t s = (hipStream_t)stream;
     if (((uintptr_t)logits & 1u) != 0) return fail(-1, "fused_sumexp launcher: pointer is not 2-byte aligned");
-    hipLaunchKernelGGL((sumexp_kernel<T>), dim3((unsigned)m), dim3(kSweepThreads), 0, s, n, (const uint16_t *)logits,
-                       (const float *)row_max, (float *)row_sum);
+    if (n > 16384)
+        hipLaunchKernelGGL((sumexp_kernel<T, 1024>), dim3((unsigned)m), dim3(1024), 0, s, n, (const uint16_t *)logits,
+                           (const float *)row_max, (float *)row_sum);
+    else
+        hipLaunchKernelGGL((sumexp_kernel<T, 256>), dim3((unsigned)m), dim3(256), 0, s, n, (const uint16_t *)logits,
+                           (const float *)row_max, (float *)row_sum);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : fail((int)e, who, e);
 }
