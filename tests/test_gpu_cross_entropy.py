@@ -339,3 +339,30 @@ def test_language_model_head_shape(m, n, name, dtype):
     assert (at_target < 0).all()
     del x, softmax
     torch.cuda.empty_cache()
+
+
+def test_more_than_2_to_the_31_logits():
+    """20,000 rows x 128,257 classes (2.57e9 elements, odd row length): rows whose element offsets lie beyond
+    2^31 and 2^32 bytes are checked against the oracle, forward and backward."""
+    m, n = 20000, 128257
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
+    for lo in range(0, m, 2000):
+        x[lo:lo + 2000] = (torch.randn(2000, n, generator=gen, device="cuda") * 2).bfloat16()
+    t = torch.randint(0, n, (m,), generator=gen, device="cuda", dtype=torch.int32)
+    softmax = torch.empty_like(x)
+    out = torch.empty(m, dtype=torch.float32, device="cuda")
+    F.cross_entropy_forward(m, n, x, t, softmax, out, -100)
+    rows = [0, 1, 8371, 8372, 16743, 16744, 16745, m - 2, m - 1]       # around 2^30 and 2^31 elements, and the end
+    idx = torch.tensor(rows, device="cuda")
+    want_soft, want_loss = oracle.ce_forward(bits16(x[idx]), t[idx].cpu().numpy(), -100, "bf16")
+    assert ulp_distance16(bits16(softmax[idx]), want_soft).max() <= 1
+    np.testing.assert_allclose(out[idx].cpu().numpy(), want_loss, rtol=2e-6, atol=2e-6)
+    assert torch.isfinite(out).all()
+    v = torch.rand(m, generator=gen, device="cuda")
+    want = bits16(softmax[idx])
+    oracle.ce_backward_inplace(v[idx].cpu().numpy(), t[idx].cpu().numpy(), want, -100, "bf16")
+    F.cross_entropy_backward_inplace(m, n, v, t, softmax, -100)
+    assert np.array_equal(bits16(softmax[idx]), want)
+    del x, softmax
+    torch.cuda.empty_cache()
