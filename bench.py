@@ -206,11 +206,12 @@ def other_workloads(torch, dev, LF, OF, iters=20):
     return out
 
 
-def tensor_list_step(torch, p16, grad, p32, mom, var, merge, iters=5):
+def tensor_list_step(torch, p16, grad, p32, mom, var, merge, batch=True, iters=5):
     """The same 6.74 B elements stepped the way a training script does it: 291 parameter tensors of the
     Llama-7B shapes (views into the flat buffers, as ZeRO keeps them; state pre-populated at step 99) through
     `AdamOptimizer.step()`.  merge = True: the optimizer finds the tensors back to back and steps them as one
-    run; merge = False: one launch per large tensor and one batched launch for the 65 norm vectors."""
+    run; merge = False: up to 32 tensors per launch, tiles handed out by ticket; batch = False as well: one
+    launch per tensor."""
     import bmtrain_amd as bmt
     layer = [(4096, 4096)] * 4 + [(11008, 4096)] * 2 + [(4096, 11008)] + [(4096,)] * 2
     shapes = [(32000, 4096)] + layer * 32 + [(4096,), (32000, 4096)]
@@ -226,6 +227,7 @@ def tensor_list_step(torch, p16, grad, p32, mom, var, merge, iters=5):
     assert lo == p16.numel()
     opt = bmt.optim.AdamOptimizer([q[0] for q in params], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
     opt.merge_adjacent = merge
+    opt.batch_launches = batch
     for param, lo, size, shape in params:
         opt.state[param] = {"step": 99, "exp_avg": mom[lo:lo + size].view(shape),
                             "exp_avg_sq": var[lo:lo + size].view(shape), "_param_fp32": p32[lo:lo + size].view(shape)}
@@ -385,7 +387,8 @@ def main():
     side = not (args.small or args.no_other_workloads)
     tensor_list = None if not side else {
         "adjacent_tensors_merged": tensor_list_step(torch, p16, grad, p32, mom, var, True),
-        "one_launch_per_tensor": tensor_list_step(torch, p16, grad, p32, mom, var, False)}
+        "32_tensors_per_launch": tensor_list_step(torch, p16, grad, p32, mom, var, False),
+        "one_launch_per_tensor": tensor_list_step(torch, p16, grad, p32, mom, var, False, batch=False)}
     # free the device before the side measurements and the host baseline
     del p32, mom, var, grad, p16, logits, softmax
     torch.cuda.empty_cache()

@@ -326,14 +326,15 @@ struct AdamBatch {
     int32_t count;
 };
 
-template <bool FP16>
-__global__ __launch_bounds__(kAdamThreads) void adam_multi_kernel(AdamBatch batch, AdamHyper h) {
+template <bool FP16, bool TICKET>
+__global__ __launch_bounds__(kAdamThreads) void adam_multi_kernel(AdamBatch batch, AdamHyper h, uint32_t *counter) {
     const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
+    const uint32_t tile = (uint32_t)adam_tile_index<TICKET>(counter);
     int t = 0;
-    while (t + 1 < batch.count && blockIdx.x >= batch.first_tile[t + 1]) t++;
+    while (t + 1 < batch.count && tile >= batch.first_tile[t + 1]) t++;
     const int64_t n = batch.n[t];
     const int64_t nvec = n / 4;
-    const int64_t i = (int64_t)(blockIdx.x - batch.first_tile[t]) * kAdamThreads + threadIdx.x;
+    const int64_t i = (int64_t)(tile - batch.first_tile[t]) * kAdamThreads + threadIdx.x;
     float *p32 = batch.p32[t];
     float *var = batch.var[t];
     uint16_t *p16 = batch.p16[t];
@@ -383,7 +384,20 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
     AdamBatch batch;
     auto flush = [&]() -> hipError_t {
         if (batch.count == 0) return hipSuccess;
-        hipLaunchKernelGGL(adam_multi_kernel<FP16>, dim3(batch.first_tile[batch.count]), dim3(kAdamThreads), 0, s, batch, h);
+        const uint32_t tiles = batch.first_tile[batch.count];
+        // Long launches hand tiles out by ticket, like the single-tensor kernels.  The counter sits in the
+        // first 16-bit output vector of the last tile of the last tensor, which the workgroup with the last
+        // ticket overwrites; a last tile that holds leftover elements only has no such vector.
+        const int last = batch.count - 1;
+        const int64_t last_first_vec = (int64_t)(tiles - 1 - batch.first_tile[last]) * kAdamThreads;
+        if ((int64_t)tiles >= kAdamTicketMinTiles && last_first_vec < batch.n[last] / 4) {
+            uint32_t *counter = (uint32_t *)((u32x2 *)batch.p16[last] + last_first_vec);
+            hipLaunchKernelGGL(adam_ticket_reset_kernel, dim3(1), dim3(1), 0, s, counter);
+            hipLaunchKernelGGL((adam_multi_kernel<FP16, true>), dim3(tiles), dim3(kAdamThreads), 0, s, batch, h, counter);
+        } else {
+            hipLaunchKernelGGL((adam_multi_kernel<FP16, false>), dim3(tiles), dim3(kAdamThreads), 0, s, batch, h,
+                               (uint32_t *)nullptr);
+        }
         batch.count = 0;
         batch.first_tile[0] = 0;
         return hipGetLastError();

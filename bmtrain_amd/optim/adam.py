@@ -42,9 +42,11 @@ class AdamOptimizer(torch.optim.Optimizer):
         self._hold_steps = hold_steps
         # Tensors below `batch_below` elements share launches (same arithmetic per element as one launch per
         # tensor, which remains available by setting batch_launches to False).  Larger tensors keep a launch
-        # of their own: they stream at full rate either way, and slightly faster alone.
+        # of their own unless the tensors that could share launches hold `batch_all_from` elements or more.
         self.batch_launches = True
         self.batch_below = 1 << 20
+        self.batch_all_from = 1 << 26
+        self.ticket_alone = 1 << 28
         # Parameters, gradients and state that are adjacent in memory are stepped as one flat tensor.
         self.merge_adjacent = True
 
@@ -124,19 +126,30 @@ class AdamOptimizer(torch.optim.Optimizer):
                     lr = 0.0 if state["step"] < self._hold_steps else group["lr"]
                     half.append((state["_param_fp32"], p, grad, state["exp_avg"], state["exp_avg_sq"], state["step"], lr))
 
-            # 16-bit parameters that can share launches: (dtype, step, lr) -> tensors
-            batches = {}
+            # 16-bit parameters that can share launches: (dtype, step, lr) -> tensors.  Small tensors always
+            # do; when a class holds enough elements for tiles to be handed out by ticket (where one long
+            # launch beats many medium ones), the large tensors join it too.
+            batches, singles = {}, []
             for run in _adjacent_runs(half) if self.merge_adjacent else [[w] for w in half]:
                 p32, p, grad, m, v, step, lr = run[0]
                 if len(run) > 1:
                     total = sum(w[1].numel() for w in run)
                     p32, p, grad, m, v = (t.as_strided((total,), (1,)) for t in (p32, p, grad, m, v))
-                elif (self.batch_launches and p.numel() < self.batch_below and p.is_contiguous()
-                        and grad.is_contiguous()):
-                    batches.setdefault((p.dtype, step, lr), []).append((p32, p, grad, m, v))
-                    continue
+                item = (p32, p, grad, m, v, step, lr)
+                if self.batch_launches and p.is_contiguous() and grad.is_contiguous():
+                    batches.setdefault((p.dtype, step, lr), []).append(item)
+                else:
+                    singles.append(item)
+            for key in list(batches):
+                # tensors of `ticket_alone` elements or more are long launches by themselves
+                shared = [w for w in batches[key] if w[1].numel() < self.ticket_alone]
+                limit = self.ticket_alone if sum(w[1].numel() for w in shared) >= self.batch_all_from else self.batch_below
+                singles.extend(w for w in batches[key] if w[1].numel() >= limit)
+                batches[key] = [w for w in batches[key] if w[1].numel() < limit]
+            for p32, p, grad, m, v, step, lr in singles:
                 fused = F.adam_fp16 if p.dtype == torch.float16 else F.adam_bf16
                 fused(p32, p, grad, m, v, beta1, beta2, group["eps"], lr, scale, group["weight_decay"], step)
+            batches = {key: [w[:5] for w in items] for key, items in batches.items() if items}
             for (_, step, lr), tensors in batches.items():
                 F.adam_multi(tensors, beta1, beta2, group["eps"], lr, scale, group["weight_decay"], step)
         return loss

@@ -343,6 +343,33 @@ def test_multi_tensor_launch_equals_per_tensor_launches(flavour):
         F.adam_multi([(single[0][0], single[0][1].float(), single[0][2], single[0][3], single[0][4])], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.0, 1)
 
 
+@pytest.mark.parametrize("flavour", ["bf16", "fp16"])
+def test_long_multi_tensor_launch_hands_tiles_out_by_ticket(flavour):
+    """Batches of 8,192 tiles or more draw tiles from a counter kept in the last tensor's 16-bit output.
+    40 tensors (two launches), bit for bit against one launch per tensor; a second table ends in a tensor
+    whose last tile holds leftover elements only (no room for the counter: workgroup-id order)."""
+    dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
+    mdt = torch.float16 if flavour == "fp16" else torch.float32
+    fn = F.adam_fp16 if flavour == "fp16" else F.adam_bf16
+    for sizes in ([1_200_001 + 4 * k for k in range(39)] + [2_000_003], [1_200_000] * 32 + [4096 * 300 + 3]):
+        gen = torch.Generator(device="cuda").manual_seed(len(sizes))
+        single, multi = [], []
+        for n in sizes:
+            p = torch.randn(n, generator=gen, device="cuda") * 0.02
+            m = (torch.randn(n, generator=gen, device="cuda") * 1e-4).to(mdt)
+            v = (torch.randn(n, generator=gen, device="cuda") * 1e-6).abs()
+            g = (torch.randn(n, generator=gen, device="cuda") * 1e-3).to(dt16)
+            for dest in (single, multi):
+                dest.append((p.clone(), torch.full((n,), -1, dtype=dt16, device="cuda"), g, m.clone(), v.clone()))
+        for p32, p16, g, m, v in single:
+            fn(p32, p16, g, m, v, 0.9, 0.999, 1e-8, 1e-3, 2.0, 0.01, 5)
+        F.adam_multi(multi, 0.9, 0.999, 1e-8, 1e-3, 2.0, 0.01, 5)
+        for a, b in zip(single, multi):
+            for x, y in zip(a, b):
+                assert torch.equal(x.view(torch.int16 if x.element_size() == 2 else torch.int32),
+                                   y.view(torch.int16 if y.element_size() == 2 else torch.int32))
+
+
 def _checksum(t, chunk=1 << 28):
     """Order-independent 64-bit checksum of a tensor's bit patterns."""
     view = t.view(torch.int32 if t.element_size() == 4 else torch.int16)
