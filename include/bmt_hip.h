@@ -148,6 +148,8 @@ BMT_API int fused_softmax_inplace_bf16_launcher(int32_t m, int32_t n, void *logi
  * `count` tensors that share their hyper-parameters (same group, same step count) in as few launches as
  * possible; per element the arithmetic is that of adam_{fp16,bf16}_launcher, bit for bit.
  * `tensors` is a host array; `m` is float[n] for bf16 and half[n] for fp16.  Entries with n <= 0 are skipped.
+ * param_16 is output only; a launch over 2^25 elements or more keeps a tile counter in 4 bytes of the
+ * last tensor's param_16 while it runs.
  */
 typedef struct bmt_adam_tensor {
     void *param_fp32;
