@@ -114,21 +114,35 @@ def cpu_baseline():
         "ms_per_step": round(median * 1e3, 3),
         "elements_per_s": round(n / median, 1),
     }
+    # the reference's bf16 host path (a scalar loop per thread), same inputs, 10 steps
+    if ref is not None:
+        gb = [(torch.randn(n, generator=gen) * 1e-3).bfloat16().view(torch.int16).numpy().view(np.uint16).copy()]
+        bf_times = []
+        for k in range(10):
+            bc1, bc2 = oracle.bias_corrections(0.9, 0.999, k + 1)
+            t0 = time.perf_counter()
+            ref.adam_cpu_bf16_launcher(n, p.ctypes.data, h.ctypes.data, 0, gb[0].ctypes.data, m.ctypes.data,
+                                       v.ctypes.data, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, bc1, bc2)
+            bf_times.append(time.perf_counter() - t0)
+        bf_times.sort()
+        out["adam_bf16_GBps"] = round(ADAM_BF16_BYTES * n / bf_times[5] / 1e9, 3)
+        out["adam_bf16_sample"] = f"adam_cpu bf16 grads, N=2^24, 10 steps, median {bf_times[5] * 1e3:.2f} ms/step"
     # CPU cross-entropy (torch), fp32 as FusedCrossEntropy itself does for fp32 input
     torch.set_num_threads(cores)
-    rows, classes = 256, 128256
-    x = (torch.randn(rows, classes, generator=gen) * 3).requires_grad_()
-    t = torch.randint(0, classes, (rows,), generator=gen)
-    t[::20] = -100
-    best = float("inf")
-    for _ in range(3):
-        x.grad = None
-        t0 = time.perf_counter()
-        loss = torch.nn.functional.cross_entropy(x, t, ignore_index=-100)
-        loss.backward()
-        best = min(best, time.perf_counter() - t0)
-    out["ce_rows_per_s"] = round(rows / best, 1)
-    out["ce_sample"] = f"torch CPU cross_entropy fwd+bwd fp32, {rows} rows x {classes} classes, {cores} threads, best of 3"
+    for key, rows, classes, std, every in (("ce", 256, 128256, 3.0, 20), ("ce_32000", 1024, 32000, 2.0, 10)):
+        x = (torch.randn(rows, classes, generator=gen) * std).requires_grad_()
+        t = torch.randint(0, classes, (rows,), generator=gen)
+        t[::every] = -100
+        best = float("inf")
+        for _ in range(3):
+            x.grad = None
+            t0 = time.perf_counter()
+            loss = torch.nn.functional.cross_entropy(x, t, ignore_index=-100)
+            loss.backward()
+            best = min(best, time.perf_counter() - t0)
+        out[key + "_rows_per_s"] = round(rows / best, 1)
+        out[key + "_sample"] = (f"torch CPU cross_entropy fwd+bwd fp32, {rows} rows x {classes} classes, "
+                                f"{cores} threads, best of 3")
     return out
 
 
