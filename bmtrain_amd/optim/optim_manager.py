@@ -15,13 +15,27 @@ from ._base import flat_runs
 from ._function import grad_stats
 
 
-def check_overflow(param_groups):
+def _scanned_grads(param_groups):
+    """The gradients the overflow check looks at: those of non-fp32 parameters."""
+    return [p.grad for group in param_groups for p in group["params"] if p.grad is not None and p.dtype != torch.float]
+
+
+def _fingerprint(g):
+    """Identifies a gradient's memory and its contents' version (in-place writes bump the counter)."""
+    return (g.data_ptr(), g.numel(), g.dtype, g._version)
+
+
+def check_overflow(param_groups, known=None):
     """Raises OverflowError when any non-fp32 gradient holds an inf or NaN
-    (optim_manager.py:9-21)."""
-    flag = torch.zeros(1, dtype=torch.uint8, device="cuda")[0]
-    grads = [p.grad for group in param_groups for p in group["params"] if p.grad is not None and p.dtype != torch.float]
-    for g in flat_runs(grads):      # gradients that lie back to back are scanned by one launch
-        has_inf_nan(g, flag)
+    (optim_manager.py:9-21).  `known` may carry the verdict of an earlier pass over gradients:
+    a pair (flag tensor, {fingerprint}); gradients found in it unchanged are not read again."""
+    grads = _scanned_grads(param_groups)
+    if known is not None and all(_fingerprint(g) in known[1] for g in grads):
+        flag = known[0]
+    else:
+        flag = torch.zeros(1, dtype=torch.uint8, device="cuda")[0]
+        for g in flat_runs(grads):      # gradients that lie back to back are scanned by one launch
+            has_inf_nan(g, flag)
     if flag > 0:
         raise OverflowError("Gradient overflow")
 
@@ -54,6 +68,8 @@ class OptimManager:
         self.grad_scale = config["zero_size"] if grad_scale is None else grad_scale
         self.optimizers = []
         self.lr_schedulers = []
+        # verdict of the overflow scan that clip_grad_norm's pass over the gradients produced on the side
+        self._known_overflow = None
 
     def add_optimizer(self, optimizer: torch.optim.Optimizer, lr_scheduler=None):
         """All optimizers of one manager share the loss scale."""
@@ -77,19 +93,23 @@ class OptimManager:
             current.wait_stream(load_stream)
 
     def backward(self, loss: torch.Tensor):
+        self._known_overflow = None
         self.scale_loss(loss).backward()
         self._join_load_stream(after_step=False)
 
     def zero_grad(self):
+        self._known_overflow = None
         for optimizer in self.optimizers:
             optimizer.zero_grad(set_to_none=False)
 
     def _overflowed(self) -> bool:
         for optimizer in self.optimizers:
             try:
-                check_overflow(optimizer.param_groups)
+                check_overflow(optimizer.param_groups, self._known_overflow)
             except OverflowError:
+                self._known_overflow = None
                 return True
+        self._known_overflow = None
         return False
 
     def step(self):
@@ -122,6 +142,7 @@ class OptimManager:
         """Clips the (still loss-scaled) gradients to ``max_norm`` in place and returns the
         unscaled total norm (optim_manager.py:158-200)."""
         scale = self.loss_scale
+        scanned = None
         parameters = [p for group in param_groups for p in group["params"]]
         grads = [p.grad.data if p.grad is not None else torch.zeros_like(p.data) for p in parameters]
         if norm_type == "inf":
@@ -139,6 +160,8 @@ class OptimManager:
                 for g in flat_runs(fused):
                     grad_stats(g, sumsq, flag)
                 acc += sumsq.float()
+                fused_ids = {id(g) for g in fused}
+                scanned = (flag, [p.grad for p, g in zip(parameters, grads) if id(g) in fused_ids])
             fused_ids = {id(g) for g in fused}
             for g in grads:
                 if id(g) not in fused_ids:
@@ -149,6 +172,12 @@ class OptimManager:
             for p in parameters:
                 if p.grad is not None:
                     p.grad.data.mul_(clip_coef)
+        # The pass over the 16-bit gradients also looked for inf / NaN, and the scaling above cannot change that
+        # verdict (it multiplies by a finite factor below one, or by zero when the norm itself is infinite);
+        # step() reuses it for gradients that nobody has written to since.
+        self._known_overflow = None
+        if scanned is not None:
+            self._known_overflow = (scanned[0][0], {_fingerprint(g) for g in scanned[1]})
         return total_norm / scale
 
     @torch.no_grad()

@@ -208,6 +208,47 @@ def test_overflow_check_and_grad_norm_over_flat_gradient_storage():
         check_overflow(groups)
 
 
+def test_step_reuses_the_overflow_verdict_of_the_clipping_pass(monkeypatch):
+    """clip_grad_norm reads the 16-bit gradients once for norm and overflow flag; step() does not scan gradients
+    nobody has written to since, and does scan again after any in-place write."""
+    import bmtrain_amd.optim.optim_manager as om
+    calls = []
+    real = om.has_inf_nan
+    monkeypatch.setattr(om, "has_inf_nan", lambda g, flag: (calls.append(g.numel()), real(g, flag))[1])
+    torch.manual_seed(8)
+    ps = [torch.nn.Parameter(torch.randn(s, device="cuda").bfloat16()) for s in (5000, 77, 4096)]
+    opt = bmt.optim.AdamOptimizer(ps, lr=1e-3)
+    manager = bmt.optim.OptimManager(loss_scale=64, loss_scale_steps=1000)
+    manager.add_optimizer(opt)
+
+    def grads():
+        for p in ps:
+            p.grad = (torch.randn_like(p.float()) * 64).bfloat16()
+
+    grads()
+    manager.clip_grad_norm(opt.param_groups, max_norm=0.5)          # clips: gradients are scaled in place
+    manager.step()
+    assert calls == [] and opt.state[ps[0]]["step"] == 1             # verdict reused, step taken
+    grads()
+    manager.step()
+    assert len(calls) == 3                                           # no clipping pass: scanned as usual
+    calls.clear(); grads()
+    manager.clip_grad_norm(opt.param_groups, max_norm=1e9)
+    ps[1].grad.mul_(2.0)                                             # somebody writes to a gradient
+    manager.step()
+    assert len(calls) == 3 and opt.state[ps[0]]["step"] == 3
+    calls.clear(); grads()
+    ps[2].grad[100] = float("nan")
+    manager.clip_grad_norm(opt.param_groups, max_norm=1.0)
+    manager.step()                                                   # overflow seen by the clipping pass
+    assert calls == [] and manager.loss_scale == 32 and opt.state[ps[0]]["step"] == 3
+    calls.clear(); grads()
+    manager.clip_grad_norm([{"params": ps[:2]}], max_norm=1.0)      # a subset only: the rest must be scanned
+    ps[2].grad[5] = float("inf")
+    manager.step()
+    assert len(calls) == 3 and manager.loss_scale == 16
+
+
 def test_overflow_skips_the_step_and_halves_the_scale():
     torch.manual_seed(2)
     p = torch.nn.Parameter(torch.randn(1000, device="cuda").half())
