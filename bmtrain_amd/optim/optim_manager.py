@@ -169,9 +169,8 @@ class OptimManager:
             total_norm = acc[0] ** (1.0 / norm_type)
         clip_coef = float(max_norm * scale) / (total_norm + eps)
         if clip_coef < 1:
-            for p in parameters:
-                if p.grad is not None:
-                    p.grad.data.mul_(clip_coef)
+            for g in flat_runs([p.grad.data for p in parameters if p.grad is not None]):
+                g.mul_(clip_coef)      # back-to-back gradients are scaled by one launch
         # The pass over the 16-bit gradients also looked for inf / NaN, and the scaling above cannot change that
         # verdict (it multiplies by a finite factor below one, or by zero when the norm itself is infinite);
         # step() reuses it for gradients that nobody has written to since.
