@@ -199,6 +199,13 @@ def test_overflow_check_and_grad_norm_over_flat_gradient_storage():
     want = torch.cat([flat_g.float(), lone.grad.float()]).norm() / 64
     got = manager.clip_grad_norm(groups, max_norm=1e9)
     torch.testing.assert_close(got, want, rtol=1e-5, atol=0)
+    before = flat_g.clone()
+    got = manager.clip_grad_norm(groups, max_norm=0.25)      # clips: the whole run is scaled by one launch
+    coef = (0.25 * 64) / (want * 64 + 1e-6)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=0)
+    assert torch.equal(flat_g, (before.float() * coef).bfloat16()) or \
+        ((flat_g.float() - before.float() * coef).abs() <= before.float().abs() * coef * 2.0 ** -7).all()
+    assert torch.equal(lone.grad, (torch.ones(33, device="cuda") * coef).half())
     flat_g[4096 + 7 + 50000] = float("nan")                  # inside the third tensor of the run
     with pytest.raises(OverflowError):
         check_overflow(groups)
