@@ -96,16 +96,18 @@ class AdamTensor(ctypes.Structure):
     _fields_ = [("param_fp32", _p), ("param_16", _p), ("grad_16", _p), ("m", _p), ("v", _p), ("n", _i64)]
 
 
-def _bind_multi(name):
+def _bind_multi(name, extra_floats=0):
     fn = getattr(_lib, name)
-    fn.argtypes = [_i32, ctypes.POINTER(AdamTensor)] + _HYPER + [_p]
+    fn.argtypes = [_i32, ctypes.POINTER(AdamTensor)] + _HYPER + [_f] * extra_floats + [_p]
     fn.restype = ctypes.c_int
 
-    def call(tensors, beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2, stream):
-        """tensors: sequence of (param_fp32_ptr, param_16_ptr, grad_16_ptr, m_ptr, v_ptr, n)."""
+    def call(tensors, *args):
+        """tensors: sequence of (param_fp32_ptr, param_16_ptr, grad_16_ptr, m_ptr, v_ptr, n); then beta1, beta2,
+        eps, lr, scale, weight_decay, bias_correction1, bias_correction2[, grad_coef], stream."""
+        if len(args) != len(_HYPER) + extra_floats + 1:
+            raise TypeError(f"{name}() takes {len(_HYPER) + extra_floats + 2} positional arguments")
         table = (AdamTensor * len(tensors))(*[AdamTensor(*t) for t in tensors])
-        status = fn(len(tensors), table, beta1, beta2, eps, lr, scale, weight_decay, bias_correction1,
-                    bias_correction2, stream)
+        status = fn(len(tensors), table, *args)
         if status != 0:
             raise RuntimeError(f"{name} failed with status {status}: {last_error()}")
 
@@ -115,6 +117,9 @@ def _bind_multi(name):
 
 adam_bf16_multi_launcher = _bind_multi("adam_bf16_multi_launcher")
 adam_fp16_multi_launcher = _bind_multi("adam_fp16_multi_launcher")
+adam_bf16_multi_clip_launcher = _bind_multi("adam_bf16_multi_clip_launcher", 1)
+adam_fp16_multi_clip_launcher = _bind_multi("adam_fp16_multi_clip_launcher", 1)
 
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["is_bf16_supported", "bmt_hip_last_error", "grad_stats_workspace_floats",
-                                                  "adam_bf16_multi_launcher", "adam_fp16_multi_launcher"])
+                                                  "adam_bf16_multi_launcher", "adam_fp16_multi_launcher",
+                                                  "adam_bf16_multi_clip_launcher", "adam_fp16_multi_clip_launcher"])

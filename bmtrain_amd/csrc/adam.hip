@@ -31,7 +31,17 @@ namespace bmt {
 
 struct AdamHyper {
     float b1, b2, eps, lr, scale, wd, bc1, bc2;
+    float gcoef = 1.0f;   // gradient clipping factor applied on the fly (1: none), see clip16
 };
+
+// Gradient clipping folded into the step.  Eagerly, clipping multiplies the 16-bit gradient in
+// place: fp32 product of the gradient and the (16-bit-rounded) factor, rounded back to 16 bits.
+// Doing exactly that to the value in flight gives the same bits without the extra pass over the
+// gradients.
+template <typename T>
+__device__ __forceinline__ float clip16(float g, float coef) {
+    return coef == 1.0f ? g : T::to_f32(T::from_f32(g * coef));
+}
 
 // Per-element update, bf16 flavour (plain fp32 moments).
 __device__ __forceinline__ void adam_elem_unscaled(float g16f, float &m, float &v, float &p, const AdamHyper &h,
@@ -63,7 +73,7 @@ __device__ __forceinline__ void adam_group_unscaled(u32x2 g, f32x4 &m, f32x4 &v,
     float gm[4] = {lo_f32<T>(g.x), hi_f32<T>(g.x), lo_f32<T>(g.y), hi_f32<T>(g.y)};
     float ma[4] = {m.x, m.y, m.z, m.w}, va[4] = {v.x, v.y, v.z, v.w}, pa[4] = {p.x, p.y, p.z, p.w};
 #pragma unroll
-    for (int k = 0; k < 4; k++) adam_elem_unscaled(gm[k], ma[k], va[k], pa[k], h, omb1, omb2, lrwd);
+    for (int k = 0; k < 4; k++) adam_elem_unscaled(clip16<T>(gm[k], h.gcoef), ma[k], va[k], pa[k], h, omb1, omb2, lrwd);
     m = f32x4{ma[0], ma[1], ma[2], ma[3]};
     v = f32x4{va[0], va[1], va[2], va[3]};
     p = f32x4{pa[0], pa[1], pa[2], pa[3]};
@@ -74,7 +84,7 @@ __device__ __forceinline__ void adam_group_scaled(u32x2 g, f32x4 &m, f32x4 &v, f
     float gm[4] = {lo_f32<T>(g.x), hi_f32<T>(g.x), lo_f32<T>(g.y), hi_f32<T>(g.y)};
     float ma[4] = {m.x, m.y, m.z, m.w}, va[4] = {v.x, v.y, v.z, v.w}, pa[4] = {p.x, p.y, p.z, p.w};
 #pragma unroll
-    for (int k = 0; k < 4; k++) adam_elem_scaled(gm[k], ma[k], va[k], pa[k], h, omb1, omb2, lrwd, eps_s);
+    for (int k = 0; k < 4; k++) adam_elem_scaled(clip16<T>(gm[k], h.gcoef), ma[k], va[k], pa[k], h, omb1, omb2, lrwd, eps_s);
     m = f32x4{ma[0], ma[1], ma[2], ma[3]};
     v = f32x4{va[0], va[1], va[2], va[3]};
     p = f32x4{pa[0], pa[1], pa[2], pa[3]};
@@ -186,7 +196,7 @@ __global__ __launch_bounds__(kAdamScalarThreads) void adam_bf16_scalar_kernel(
     for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < total; k += (int64_t)gridDim.x * blockDim.x) {
         const int64_t i = k < n0 ? lo0 + k : lo1 + (k - n0);
         float p = p32[i], m = mom[i], v = var[i];
-        adam_elem_unscaled(BFloat16::to_f32(g16[i]), m, v, p, h, omb1, omb2, lrwd);
+        adam_elem_unscaled(clip16<BFloat16>(BFloat16::to_f32(g16[i]), h.gcoef), m, v, p, h, omb1, omb2, lrwd);
         p32[i] = p; mom[i] = m; var[i] = v; p16[i] = BFloat16::from_f32(p);
     }
 }
@@ -198,7 +208,7 @@ __global__ __launch_bounds__(kAdamScalarThreads) void adam_fp16_scalar_kernel(
     for (int64_t k = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; k < total; k += (int64_t)gridDim.x * blockDim.x) {
         const int64_t i = k < n0 ? lo0 + k : lo1 + (k - n0);
         float p = p32[i], m = Half::to_f32(mom[i]), v = var[i];
-        adam_elem_scaled(Half::to_f32(g16[i]), m, v, p, h, omb1, omb2, lrwd, eps_s);
+        adam_elem_scaled(clip16<Half>(Half::to_f32(g16[i]), h.gcoef), m, v, p, h, omb1, omb2, lrwd, eps_s);
         p32[i] = p; mom[i] = Half::from_f32(m); var[i] = v; p16[i] = Half::from_f32(p);
     }
 }
@@ -362,12 +372,12 @@ __global__ __launch_bounds__(kAdamThreads) void adam_multi_kernel(AdamBatch batc
         if (FP16) {
             uint16_t *mom = (uint16_t *)batch.mom[t];
             float m = Half::to_f32(mom[e]);
-            adam_elem_scaled(Half::to_f32(g16[e]), m, v, p, h, omb1, omb2, lrwd, eps_s);
+            adam_elem_scaled(clip16<Half>(Half::to_f32(g16[e]), h.gcoef), m, v, p, h, omb1, omb2, lrwd, eps_s);
             mom[e] = Half::from_f32(m); p16[e] = Half::from_f32(p);
         } else {
             float *mom = (float *)batch.mom[t];
             float m = mom[e];
-            adam_elem_unscaled(BFloat16::to_f32(g16[e]), m, v, p, h, omb1, omb2, lrwd);
+            adam_elem_unscaled(clip16<BFloat16>(BFloat16::to_f32(g16[e]), h.gcoef), m, v, p, h, omb1, omb2, lrwd);
             mom[e] = m; p16[e] = BFloat16::from_f32(p);
         }
         p32[e] = p; var[e] = v;
@@ -471,4 +481,19 @@ extern "C" int adam_fp16_multi_launcher(int32_t count, const bmt_adam_tensor *te
                                         float bias_correction2, void *stream) {
     AdamHyper h{beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2};
     return adam_multi<true>(count, tensors, h, (hipStream_t)stream, "adam_fp16_multi_launcher");
+}
+
+extern "C" int adam_bf16_multi_clip_launcher(int32_t count, const bmt_adam_tensor *tensors, float beta1, float beta2,
+                                             float eps, float lr, float scale, float weight_decay,
+                                             float bias_correction1, float bias_correction2, float grad_coef,
+                                             void *stream) {
+    AdamHyper h{beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2, grad_coef};
+    return adam_multi<false>(count, tensors, h, (hipStream_t)stream, "adam_bf16_multi_clip_launcher");
+}
+extern "C" int adam_fp16_multi_clip_launcher(int32_t count, const bmt_adam_tensor *tensors, float beta1, float beta2,
+                                             float eps, float lr, float scale, float weight_decay,
+                                             float bias_correction1, float bias_correction2, float grad_coef,
+                                             void *stream) {
+    AdamHyper h{beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2, grad_coef};
+    return adam_multi<true>(count, tensors, h, (hipStream_t)stream, "adam_fp16_multi_clip_launcher");
 }

@@ -142,8 +142,11 @@ def grad_stats(g_half: torch.Tensor, sumsq: torch.Tensor, flag: torch.Tensor) ->
 
 
 def adam_multi(tensors, beta1: float, beta2: float, eps: float, lr: float, scale: float, weight_decay: float,
-               step: int) -> None:
+               step: int, grad_coef: float = 1.0) -> None:
     """Fused GPU step over several parameter tensors that share hyper-parameters and step count.
+    ``grad_coef`` != 1 applies gradient clipping on the fly: every gradient element enters the step as
+    ``to16(float(g) * grad_coef)`` — the bits an eager ``g.mul_(coef)`` would have left — while the gradient
+    tensors stay as they are.
 
     ``tensors`` is a list of ``(param_fp32, param_16, g_16, m, v_fp32)`` as ``adam_fp16`` / ``adam_bf16`` take
     them, all of one 16-bit flavour.  Same arithmetic per element; the tensors travel to the device in the
@@ -168,7 +171,10 @@ def adam_multi(tensors, beta1: float, beta2: float, eps: float, lr: float, scale
     bias_correction2 = 1 - beta2 ** step
     if flavour == torch.bfloat16:
         _require_bf16()
-        launcher = C.adam_bf16_multi_launcher
+    if grad_coef == 1.0:
+        launcher = C.adam_bf16_multi_launcher if flavour == torch.bfloat16 else C.adam_fp16_multi_launcher
+        launcher(rows, beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2, _current_stream())
     else:
-        launcher = C.adam_fp16_multi_launcher
-    launcher(rows, beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2, _current_stream())
+        launcher = C.adam_bf16_multi_clip_launcher if flavour == torch.bfloat16 else C.adam_fp16_multi_clip_launcher
+        launcher(rows, beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2, grad_coef,
+                 _current_stream())

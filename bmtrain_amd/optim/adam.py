@@ -94,9 +94,15 @@ class AdamOptimizer(torch.optim.Optimizer):
                     state["_param_fp32"].copy_(q)
                 lo = hi
 
+    # step() can apply a gradient clipping factor on the fly (see OptimManager(defer_clip=True))
+    supports_grad_coef = True
+
     @torch.no_grad()
-    def step(self, closure=None, scale=1):
-        """One optimisation step; ``scale`` is the loss scale the gradients carry."""
+    def step(self, closure=None, scale=1, grad_coef=None):
+        """One optimisation step; ``scale`` is the loss scale the gradients carry.  ``grad_coef`` (a 0-dim
+        tensor or float below one) clips on the fly: each gradient enters as if it had been multiplied in
+        place by it — for 16-bit gradients with the factor rounded to their dtype and the product rounded
+        back, as the in-place multiplication does on the GPU — but the gradient tensors are left alone."""
         loss = None
         if closure is not None:
             with torch.enable_grad():
@@ -116,6 +122,8 @@ class AdamOptimizer(torch.optim.Optimizer):
                 if p.dtype == torch.float32:
                     # hold_steps is tested before the increment on this path (adam.py:137).
                     lr = 0.0 if state["step"] < self._hold_steps else group["lr"]
+                    if grad_coef is not None:
+                        grad = grad * grad_coef
                     torch_adam_fp32(p, grad / scale, state["exp_avg"], state["exp_avg_sq"], state["step"],
                                     beta1=beta1, beta2=beta2, lr=lr, weight_decay=group["weight_decay"],
                                     eps=group["eps"])
@@ -130,28 +138,35 @@ class AdamOptimizer(torch.optim.Optimizer):
             # do; when a class holds enough elements for tiles to be handed out by ticket (where one long
             # launch beats many medium ones), the large tensors join it too.
             batches, singles = {}, []
+            coef16 = {}
+            if grad_coef is not None:      # the factor as the in-place multiplication would see it, per dtype
+                as_tensor = torch.as_tensor(grad_coef, dtype=torch.float32)
+                coef16 = {dt: float(as_tensor.to(dt).float()) for dt in (torch.float16, torch.bfloat16)}
             for run in _adjacent_runs(half) if self.merge_adjacent else [[w] for w in half]:
                 p32, p, grad, m, v, step, lr = run[0]
                 if len(run) > 1:
                     total = sum(w[1].numel() for w in run)
                     p32, p, grad, m, v = (t.as_strided((total,), (1,)) for t in (p32, p, grad, m, v))
                 item = (p32, p, grad, m, v, step, lr)
-                if self.batch_launches and p.is_contiguous() and grad.is_contiguous():
+                if (self.batch_launches or coef16) and p.is_contiguous() and grad.is_contiguous():
                     batches.setdefault((p.dtype, step, lr), []).append(item)
                 else:
                     singles.append(item)
-            for key in list(batches):
+            for key in list(batches) if not coef16 else []:     # with a clipping factor everything goes batched
                 # tensors of `ticket_alone` elements or more are long launches by themselves
                 shared = [w for w in batches[key] if w[1].numel() < self.ticket_alone]
                 limit = self.ticket_alone if sum(w[1].numel() for w in shared) >= self.batch_all_from else self.batch_below
                 singles.extend(w for w in batches[key] if w[1].numel() >= limit)
                 batches[key] = [w for w in batches[key] if w[1].numel() < limit]
             for p32, p, grad, m, v, step, lr in singles:
+                if coef16:                 # not contiguous: clip a copy of the gradient eagerly
+                    grad = grad * torch.as_tensor(grad_coef, dtype=torch.float32, device=grad.device)
                 fused = F.adam_fp16 if p.dtype == torch.float16 else F.adam_bf16
                 fused(p32, p, grad, m, v, beta1, beta2, group["eps"], lr, scale, group["weight_decay"], step)
             batches = {key: [w[:5] for w in items] for key, items in batches.items() if items}
-            for (_, step, lr), tensors in batches.items():
-                F.adam_multi(tensors, beta1, beta2, group["eps"], lr, scale, group["weight_decay"], step)
+            for (dtype, step, lr), tensors in batches.items():
+                F.adam_multi(tensors, beta1, beta2, group["eps"], lr, scale, group["weight_decay"], step,
+                             grad_coef=coef16.get(dtype, 1.0))
         return loss
 
     def get_avg_delta():

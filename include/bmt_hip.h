@@ -167,6 +167,20 @@ BMT_API int adam_fp16_multi_launcher(int32_t count, const bmt_adam_tensor *tenso
                              float bias_correction2, void *stream);
 
 /*
+ * adam_{fp16,bf16}_multi_clip_launcher — no counterpart in the reference's extension.  The same step with
+ * gradient clipping applied on the fly: every gradient element enters as to16(float(g) * grad_coef), which is
+ * what the reference's eager clipping (`p.grad.mul_(clip_coef)`, bmtrain/optim/optim_manager.py:196-199)
+ * leaves in memory when grad_coef is the clipping factor rounded to the gradient's 16-bit type; the gradients
+ * themselves are not modified.  grad_coef = 1 is the unclipped step.
+ */
+BMT_API int adam_bf16_multi_clip_launcher(int32_t count, const bmt_adam_tensor *tensors, float beta1, float beta2, float eps,
+                                  float lr, float scale, float weight_decay, float bias_correction1,
+                                  float bias_correction2, float grad_coef, void *stream);
+BMT_API int adam_fp16_multi_clip_launcher(int32_t count, const bmt_adam_tensor *tensors, float beta1, float beta2, float eps,
+                                  float lr, float scale, float weight_decay, float bias_correction1,
+                                  float bias_correction2, float grad_coef, void *stream);
+
+/*
  * grad_stats_{fp16,bf16}_launcher — no single counterpart in the reference's extension: one pass over
  * a gradient buffer that yields both quantities OptimManager needs before a step, where the reference
  * makes several (optim_manager.py:9-21 `check_overflow` via has_nan_inf_*_launcher, and :186-190

@@ -256,6 +256,63 @@ def test_step_reuses_the_overflow_verdict_of_the_clipping_pass(monkeypatch):
     assert len(calls) == 3 and manager.loss_scale == 16
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_clipping_factor_as_a_number_gives_the_bits_of_the_tensor_form(dtype):
+    """The reference clips with `g.mul_(clip_coef)`, clip_coef a 0-dim fp32 tensor on the device; torch then
+    rounds the factor to the gradient's dtype before multiplying.  The manager passes that rounded factor as a
+    Python number (a much faster kernel): the products must be the same bits."""
+    torch.manual_seed(13)
+    g = (torch.randn(1 << 18, device="cuda") * 50).to(dtype)
+    for value in (0.7368421173, 1.0 / 3.0, 0.001234567, 0.99999):
+        coef = torch.tensor(value, device="cuda")
+        assert torch.equal(g.clone().mul_(coef), g.clone().mul_(float(coef.to(dtype))))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_deferred_clipping_updates_parameters_like_eager_clipping(dtype):
+    """defer_clip: the clipping factor is applied inside the fused step.  Parameters and optimizer state end up
+    bit-identical to eager clipping (in-place multiplication of the gradients, then the step); the gradients
+    keep their unclipped values.  Mixed model: flat storage, separate tensors, an fp32 parameter."""
+    torch.manual_seed(12)
+    sizes = [4096 * 8, 77, 300001]
+    def build():
+        flat_p = (torch.randn(sum(sizes)) * 0.02).to(dtype).cuda()
+        flat_g = torch.zeros(sum(sizes), dtype=dtype, device="cuda")
+        ps, lo = [], 0
+        for size in sizes:
+            q = torch.nn.Parameter(flat_p[lo:lo + size]); q.grad = flat_g[lo:lo + size]
+            ps.append(q); lo += size
+        ps.append(torch.nn.Parameter((torch.randn(5000) * 0.02).to(dtype).cuda()))
+        ps.append(torch.nn.Parameter((torch.randn(300) * 0.02).cuda()))                # fp32
+        opt = bmt.optim.AdamOptimizer(ps, lr=1e-3, weight_decay=0.01)
+        return ps, opt
+    state = torch.get_rng_state()
+    ps_e, opt_e = build()
+    torch.set_rng_state(state)
+    ps_d, opt_d = build()
+    man_e = bmt.optim.OptimManager(loss_scale=128); man_e.add_optimizer(opt_e)
+    man_d = bmt.optim.OptimManager(loss_scale=128, defer_clip=True); man_d.add_optimizer(opt_d)
+    for step in range(3):
+        gs = [(torch.randn(p.numel(), device="cuda") * 128).to(p.dtype).view(p.shape) for p in ps_e]
+        for p, q, g in zip(ps_e, ps_d, gs):
+            if p.grad is None:
+                p.grad, q.grad = g.clone(), g.clone()
+            else:
+                p.grad.copy_(g); q.grad.copy_(g)
+        max_norm = 0.5 if step != 1 else 1e9                         # step 1 does not clip
+        n_e = man_e.clip_grad_norm(opt_e.param_groups, max_norm)
+        n_d = man_d.clip_grad_norm(opt_d.param_groups, max_norm)
+        assert torch.equal(n_e, n_d)
+        if step != 1:
+            assert not torch.equal(ps_e[0].grad, gs[0]) and torch.equal(ps_d[0].grad, gs[0])   # eager scaled, deferred not
+        man_e.step(); man_d.step()
+        for p, q in zip(ps_e, ps_d):
+            assert torch.equal(p.detach().view(torch.uint8), q.detach().view(torch.uint8)), step
+            for key in ("exp_avg", "exp_avg_sq", "_param_fp32"):
+                if key in opt_e.state[p]:
+                    assert torch.equal(opt_e.state[p][key].view(torch.uint8), opt_d.state[q][key].view(torch.uint8)), (step, key)
+
+
 def test_overflow_skips_the_step_and_halves_the_scale():
     torch.manual_seed(2)
     p = torch.nn.Parameter(torch.randn(1000, device="cuda").half())
