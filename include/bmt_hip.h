@@ -14,8 +14,9 @@
  *     never looks at the launch status.  bmt_hip_last_error() describes the last
  *     failure of the calling thread.
  *
- * Ownership: the caller owns every buffer; the library allocates nothing, keeps
- * no state between calls and retains no pointer.  GPU launchers are asynchronous
+ * Ownership: the caller owns every buffer; the library allocates no device memory,
+ * retains no pointer and keeps no state between calls apart from the host Adam's
+ * parked worker threads.  GPU launchers are asynchronous
  * on `stream` (a hipStream_t; NULL = the default stream) and never synchronise.
  * Device pointers must belong to the device that is current at the call.
  */
