@@ -353,7 +353,7 @@ def test_more_than_2_to_the_31_logits():
     softmax = torch.empty_like(x)
     out = torch.empty(m, dtype=torch.float32, device="cuda")
     F.cross_entropy_forward(m, n, x, t, softmax, out, -100)
-    rows = [0, 1, 8371, 8372, 16743, 16744, 16745, m - 2, m - 1]       # around 2^30 and 2^31 elements, and the end
+    rows = [0, 1, 8371, 8372, 16743, 16744, 16745, m - 2, m - 1]       # near 2^30 and 2^31 elements, and the end
     idx = torch.tensor(rows, device="cuda")
     want_soft, want_loss = oracle.ce_forward(bits16(x[idx]), t[idx].cpu().numpy(), -100, "bf16")
     assert ulp_distance16(bits16(softmax[idx]), want_soft).max() <= 1
