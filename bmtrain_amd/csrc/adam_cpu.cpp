@@ -29,6 +29,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <atomic>
 #include <condition_variable>
 #include <cstring>
 #include <functional>
@@ -239,7 +240,7 @@ public:
         {
             std::lock_guard<std::mutex> lock(mu_);
             stop_ = true;
-            generation_++;
+            generation_.fetch_add(1, std::memory_order_release);
         }
         wake_.notify_all();
         for (auto &t : threads_) t.join();
@@ -251,13 +252,15 @@ public:
         {
             std::lock_guard<std::mutex> lock(mu_);
             job_ = &job;
-            pending_ = (int)threads_.size();
-            generation_++;
+            pending_.store((int)threads_.size(), std::memory_order_relaxed);
+            generation_.fetch_add(1, std::memory_order_release);
         }
         wake_.notify_all();
         job(0);
+        for (int spin = 0; spin < kSpinPolls && pending_.load(std::memory_order_acquire) != 0; spin++)
+            __builtin_ia32_pause();
         std::unique_lock<std::mutex> lock(mu_);
-        done_.wait(lock, [this] { return pending_ == 0; });
+        done_.wait(lock, [this] { return pending_.load(std::memory_order_relaxed) == 0; });
         job_ = nullptr;
     }
 
@@ -266,17 +269,21 @@ private:
         uint64_t seen = 0;
         for (;;) {
             const std::function<void(int)> *job = nullptr;
+            // Calls often come in quick succession (one per piece of a tensor that is being copied in):
+            // poll for the next job for a short while before going to sleep on the condition variable.
+            for (int spin = 0; spin < kSpinPolls && generation_.load(std::memory_order_acquire) == seen; spin++)
+                __builtin_ia32_pause();
             {
                 std::unique_lock<std::mutex> lock(mu_);
-                wake_.wait(lock, [&] { return generation_ != seen; });
-                seen = generation_;
+                wake_.wait(lock, [&] { return generation_.load(std::memory_order_relaxed) != seen; });
+                seen = generation_.load(std::memory_order_relaxed);
                 if (stop_) return;
                 job = job_;
             }
             (*job)(slot);
             {
                 std::lock_guard<std::mutex> lock(mu_);
-                if (--pending_ == 0) done_.notify_one();
+                if (pending_.fetch_sub(1, std::memory_order_acq_rel) == 1) done_.notify_one();
             }
         }
     }
@@ -285,8 +292,9 @@ private:
     std::mutex mu_;
     std::condition_variable wake_, done_;
     const std::function<void(int)> *job_ = nullptr;
-    uint64_t generation_ = 0;
-    int pending_ = 0;
+    static constexpr int kSpinPolls = 200000;   // roughly a millisecond
+    std::atomic<uint64_t> generation_{0};
+    std::atomic<int> pending_{0};
     bool stop_ = false;
 };
 
