@@ -95,21 +95,12 @@ __device__ __forceinline__ T ld(const T *p) { return __builtin_nontemporal_load(
 template <typename T>
 __device__ __forceinline__ void st(T *p, T v) { __builtin_nontemporal_store(v, p); }
 
-// Launch shape of the vector kernels.  One workgroup owns one tile and exits: streaming
-// kernels on this part run faster with many short workgroups than with a resident grid that
-// loops (measured: about +5 % on a 28 B/element stream), because the dispatcher keeps every CU
-// supplied with fresh waves whose loads are all issued up front.
+// Launch shape of the short vector kernels: one workgroup owns one tile and exits.
 constexpr int kAdamThreads = 1024;
 constexpr int kAdamUnroll = 1;
 
-// Which tile a workgroup takes.  Over a long launch the eight XCDs drift apart when tiles are
-// bound to workgroup ids, and the five streams then touch widely separated DRAM pages at any one
-// time; handing tiles out in the order in which workgroups actually start keeps the accesses of
-// the whole chip within a few MiB of each other (measured: 72.6 % -> 80.2 % of HBM peak on 6.74 B
-// elements, 71 % -> 81 % on 202 M).  The ticket counter needs no workspace: it lives in the last
-// dword pair of the 16-bit parameter output, which nothing reads during the launch, is zeroed by
-// a one-lane kernel in front, and is overwritten with its real value by the workgroup that draws
-// the last ticket — after which no ticket is drawn any more.
+// The multi-tensor kernel hands its tiles out by ticket from 8,192 tiles on: a counter in the
+// caller's 16-bit output, zeroed by a one-lane kernel in front (see adam_multi).
 __global__ void adam_ticket_reset_kernel(uint32_t *counter) { *counter = 0u; }
 
 template <bool TICKET>
@@ -120,19 +111,17 @@ __device__ __forceinline__ int64_t adam_tile_index(uint32_t *counter) {
     __syncthreads();
     return ticket;
 }
-// Launches shorter than this many tiles keep the workgroup id order (the reset launch would cost
-// more than the drift does).
 constexpr int64_t kAdamTicketMinTiles = 8192;
 
 // Vector body, bf16.  `nvec` = number of 4-element groups; every pointer is aligned for its
 // vector type.  A tile is kAdamThreads * UNROLL groups; group u of a lane sits kAdamThreads groups
 // after group u-1, so each load instruction of a wave covers 64 consecutive vectors (1 KiB of fp32).
-template <int UNROLL, bool TICKET>
+template <int UNROLL>
 __global__ __launch_bounds__(kAdamThreads) void adam_bf16_vec_kernel(
     int64_t nvec, f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, const u32x2 *__restrict__ g16,
     f32x4 *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h) {
     const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd;
-    const int64_t base = adam_tile_index<TICKET>((uint32_t *)(p16 + (nvec - 1))) * (kAdamThreads * UNROLL) + threadIdx.x;
+    const int64_t base = (int64_t)blockIdx.x * (kAdamThreads * UNROLL) + threadIdx.x;
     f32x4 p[UNROLL], m[UNROLL], v[UNROLL];
     u32x2 g[UNROLL];
     bool ok[UNROLL];
@@ -155,12 +144,12 @@ __global__ __launch_bounds__(kAdamThreads) void adam_bf16_vec_kernel(
 }
 
 // Vector body, fp16: the first moment is a 16-bit array as well.
-template <int UNROLL, bool TICKET>
+template <int UNROLL>
 __global__ __launch_bounds__(kAdamThreads) void adam_fp16_vec_kernel(
     int64_t nvec, f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, const u32x2 *__restrict__ g16,
     u32x2 *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h) {
     const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
-    const int64_t base = adam_tile_index<TICKET>((uint32_t *)(p16 + (nvec - 1))) * (kAdamThreads * UNROLL) + threadIdx.x;
+    const int64_t base = (int64_t)blockIdx.x * (kAdamThreads * UNROLL) + threadIdx.x;
     f32x4 p[UNROLL], v[UNROLL];
     u32x2 g[UNROLL], mh[UNROLL];
     bool ok[UNROLL];
@@ -183,6 +172,160 @@ __global__ __launch_bounds__(kAdamThreads) void adam_fp16_vec_kernel(
         mo.x = pack2<Half>(mm.x, mm.y); mo.y = pack2<Half>(mm.z, mm.w);
         st(p32 + i, p[u]); st(var + i, v[u]); st(mom + i, mo); st(p16 + i, o);
     }
+}
+
+// ---- long launches: a resident grid that streams ---------------------------------------------
+// From kStreamMinVec 4-element groups on, the step runs as one workgroup of 256 lanes per compute
+// unit that stays resident and works through tiles of 256 groups (4 KiB of each fp32 array, the
+// granularity at which HBM channels interleave; tiles of other sizes measured up to 15 points
+// slower).  What decides the rate of this 1:1 read/write stream is how narrow the window of
+// addresses is that the whole chip touches at any moment, and how few bytes are in flight beyond
+// what hides the latency:
+//   * tiles are handed out by atomic tickets in the order in which workgroups ask for them, so
+//     all compute units work within a few MiB of each other in every array (with tiles bound to
+//     workgroup ids the eight XCDs drift apart);
+//   * a same-address atomic takes about 11 ns on this part, which would cap a launch at one tile
+//     per 11 ns; four counters in different 4 KiB blocks serve the tiles t = 4 * ticket + k
+//     (k = 0..3; workgroup w uses counter (w / 8) % 4, so every XCD feeds every counter);
+//   * each wave keeps exactly one tile of loads in flight while it computes and stores the one
+//     before (software pipeline of depth 1, two register sets); deeper prefetch, more waves per
+//     compute unit and larger tiles all measured slower;
+//   * the ticket for the tile after the next is drawn one stage ahead by lane 0 and handed to
+//     the workgroup through LDS, so nobody waits for the atomic's round trip.
+// The compiler's own wait-count insertion cannot express this pipeline (it drains the loads that
+// were just issued before the arithmetic starts), so the vector memory instructions of the loop
+// and their waits are written by hand:  `s_waitcnt vmcnt(4)` right after the four loads of the
+// next tile means "everything older has completed" — the current tile's data, the ticket drawn a
+// stage ago, and the stores of the tile before — whatever the order in which loads, stores and
+// atomics retire.  A 16-byte store is followed by `s_nop 1`: the instruction reads its data
+// registers for two more cycles, and the compiler, which pads that hazard itself for stores it
+// emits, does not see through an asm statement.
+//
+// The four counters live in the caller's 16-bit parameter output (nothing else is writable
+// without a workspace argument): word 0 of the 8-byte vectors nvec-1, nvec-513, nvec-1025 and
+// nvec-1537.  A one-workgroup kernel in front zeroes them; the lanes that own those four groups
+// step them like any other but do not store their 16-bit result; a one-workgroup kernel behind
+// derives those four vectors from the fp32 parameters just written (the 16-bit copy is by
+// definition the rounded fp32 value).  All three run on the caller's stream, so the ordering
+// between the zeroing, the atomics (performed in memory, beyond the per-XCD L2s) and the final
+// plain stores is that of kernel boundaries.
+constexpr int kStreamThreads = 256;
+constexpr int kStreamCounters = 4;
+constexpr int64_t kStreamCounterStride = 512;            // in 8-byte vectors: 4 KiB
+constexpr int64_t kStreamMinVec = (int64_t)1 << 22;      // 2^24 elements
+
+__device__ __forceinline__ bool holds_stream_counter(int64_t i, int64_t nvec) {
+    const int64_t d = nvec - 1 - i;
+    return (d & (kStreamCounterStride - 1)) == 0 && d < kStreamCounters * kStreamCounterStride;
+}
+__global__ void adam_stream_reset_kernel(u32x2 *p16, int64_t nvec) {
+    if (threadIdx.x < kStreamCounters) p16[nvec - 1 - threadIdx.x * kStreamCounterStride] = u32x2{0u, 0u};
+}
+template <typename T>
+__global__ void adam_stream_finish_kernel(const f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, int64_t nvec) {
+    if (threadIdx.x < kStreamCounters) {
+        const int64_t i = nvec - 1 - threadIdx.x * kStreamCounterStride;
+        const f32x4 p = p32[i];
+        p16[i] = u32x2{pack2<T>(p.x, p.y), pack2<T>(p.z, p.w)};
+    }
+}
+
+template <bool FP16> struct MomentVec { typedef f32x4 type; };
+template <> struct MomentVec<true> { typedef u32x2 type; };
+template <bool FP16>
+struct StreamSet {
+    f32x4 p, v;
+    typename MomentVec<FP16>::type m;
+    u32x2 g;
+    int64_t i;      // group index of this lane in the tile
+    bool ok;        // the group exists
+};
+
+__device__ __forceinline__ void stream_load(f32x4 &dst, const f32x4 *src) {
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(src) : "memory");
+}
+__device__ __forceinline__ void stream_load(u32x2 &dst, const u32x2 *src) {
+    asm volatile("global_load_dwordx2 %0, %1, off nt" : "=v"(dst) : "v"(src) : "memory");
+}
+__device__ __forceinline__ void stream_store(f32x4 *dst, const f32x4 &v) {
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(dst), "v"(v) : "memory");
+}
+__device__ __forceinline__ void stream_store(u32x2 *dst, const u32x2 &v) {
+    asm volatile("global_store_dwordx2 %0, %1, off nt" : : "v"(dst), "v"(v) : "memory");
+}
+__device__ __forceinline__ void stream_draw(uint32_t &ticket, uint32_t *counter) {
+    const uint32_t one = 1u;
+    asm volatile("global_atomic_add %0, %1, %2, off sc0" : "=v"(ticket) : "v"(counter), "v"(one) : "memory");
+}
+
+template <bool FP16>
+__global__ __launch_bounds__(kStreamThreads) void adam_stream_kernel(
+    int64_t nvec, int64_t ntiles, f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, const u32x2 *__restrict__ g16,
+    typename MomentVec<FP16>::type *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h) {
+    typedef typename MomentVec<FP16>::type mom_t;
+    typedef StreamSet<FP16> Set;
+    const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
+    __shared__ uint32_t handed[2];
+    const int which = (int)((blockIdx.x >> 3) & (kStreamCounters - 1));
+    uint32_t *counter = (uint32_t *)(p16 + (nvec - 1 - which * kStreamCounterStride));
+    if (threadIdx.x == 0) {
+        handed[0] = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        handed[1] = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    const int64_t first = (int64_t)handed[0] * kStreamCounters + which;
+    int64_t ahead = (int64_t)handed[1] * kStreamCounters + which;     // the tile after the one in flight
+    __syncthreads();
+    if (first >= ntiles) return;
+    uint32_t drawn = 0;                                               // lane 0: ticket on its way
+    if (threadIdx.x == 0) stream_draw(drawn, counter);
+
+    auto issue = [&](Set &s, int64_t tile) {
+        s.i = tile * kStreamThreads + threadIdx.x;
+        s.ok = tile < ntiles && s.i < nvec;
+        const int64_t j = s.ok ? s.i : 0;          // lanes without a group load group 0 and drop it
+        stream_load(s.g, g16 + j);
+        stream_load(s.p, p32 + j);
+        stream_load(s.m, mom + j);
+        stream_load(s.v, var + j);
+    };
+    auto finish = [&](Set &s) {
+        if (!s.ok) return;
+        u32x2 o;
+        if constexpr (FP16) {
+            f32x4 mm = f32x4{lo_f32<Half>(s.m.x), hi_f32<Half>(s.m.x), lo_f32<Half>(s.m.y), hi_f32<Half>(s.m.y)};
+            adam_group_scaled<Half>(s.g, mm, s.v, s.p, h, omb1, omb2, lrwd, eps_s);
+            s.m = u32x2{pack2<Half>(mm.x, mm.y), pack2<Half>(mm.z, mm.w)};
+            o = u32x2{pack2<Half>(s.p.x, s.p.y), pack2<Half>(s.p.z, s.p.w)};
+        } else {
+            adam_group_unscaled<BFloat16>(s.g, s.m, s.v, s.p, h, omb1, omb2, lrwd);
+            o = u32x2{pack2<BFloat16>(s.p.x, s.p.y), pack2<BFloat16>(s.p.z, s.p.w)};
+        }
+        stream_store(p32 + s.i, s.p);
+        stream_store(mom + s.i, s.m);
+        stream_store(var + s.i, s.v);
+        if (!holds_stream_counter(s.i, nvec)) stream_store(p16 + s.i, o);
+    };
+    // One stage: the loads of the tile after `cur` go out, then `cur` is computed and stored.
+    // Returns the tile whose loads went out.
+    auto stage = [&](Set &cur, Set &next, int slot) -> int64_t {
+        const int64_t tile = ahead;
+        issue(next, tile);
+        asm volatile("s_waitcnt vmcnt(4)" : "+v"(cur.g), "+v"(cur.p), "+v"(cur.m), "+v"(cur.v), "+v"(drawn));
+        if (threadIdx.x == 0) handed[slot] = drawn;
+        __syncthreads();
+        ahead = (int64_t)handed[slot] * kStreamCounters + which;
+        if (threadIdx.x == 0) stream_draw(drawn, counter);
+        finish(cur);
+        return tile;
+    };
+    Set a, b;
+    issue(a, first);
+    while (true) {
+        if (stage(a, b, 0) >= ntiles) break;
+        if (stage(b, a, 1) >= ntiles) break;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");   // loads of the tile nobody owns, the last ticket
 }
 
 constexpr int kAdamScalarThreads = 256;
@@ -272,13 +415,16 @@ static hipError_t launch_bf16(int64_t n, float *p32, uint16_t *p16, const uint16
         n, vectorisable, head, nvec,
         [&](unsigned grid) {
             u32x2 *out16 = (u32x2 *)(p16 + head);
-            if ((int64_t)grid >= kAdamTicketMinTiles) {
-                hipLaunchKernelGGL(adam_ticket_reset_kernel, dim3(1), dim3(1), 0, s, (uint32_t *)(out16 + (nvec - 1)));
-                hipLaunchKernelGGL((adam_bf16_vec_kernel<kAdamUnroll, true>), dim3(grid), dim3(kAdamThreads), 0, s, nvec,
-                                   (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (f32x4 *)(m + head),
+            if (nvec >= kStreamMinVec) {
+                const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
+                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec);
+                hipLaunchKernelGGL((adam_stream_kernel<false>), dim3((unsigned)device_cu_count()), dim3(kStreamThreads), 0, s, nvec,
+                                   ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (f32x4 *)(m + head),
                                    (f32x4 *)(v + head), h);
+                hipLaunchKernelGGL((adam_stream_finish_kernel<BFloat16>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
+                                   out16, nvec);
             } else {
-                hipLaunchKernelGGL((adam_bf16_vec_kernel<kAdamUnroll, false>), dim3(grid), dim3(kAdamThreads), 0, s, nvec,
+                hipLaunchKernelGGL((adam_bf16_vec_kernel<kAdamUnroll>), dim3(grid), dim3(kAdamThreads), 0, s, nvec,
                                    (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (f32x4 *)(m + head),
                                    (f32x4 *)(v + head), h);
             }
@@ -299,13 +445,16 @@ static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16
         n, vectorisable, head, nvec,
         [&](unsigned grid) {
             u32x2 *out16 = (u32x2 *)(p16 + head);
-            if ((int64_t)grid >= kAdamTicketMinTiles) {
-                hipLaunchKernelGGL(adam_ticket_reset_kernel, dim3(1), dim3(1), 0, s, (uint32_t *)(out16 + (nvec - 1)));
-                hipLaunchKernelGGL((adam_fp16_vec_kernel<kAdamUnroll, true>), dim3(grid), dim3(kAdamThreads), 0, s, nvec,
-                                   (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
+            if (nvec >= kStreamMinVec) {
+                const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
+                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec);
+                hipLaunchKernelGGL((adam_stream_kernel<true>), dim3((unsigned)device_cu_count()), dim3(kStreamThreads), 0, s, nvec,
+                                   ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
                                    (f32x4 *)(v + head), h);
+                hipLaunchKernelGGL((adam_stream_finish_kernel<Half>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
+                                   out16, nvec);
             } else {
-                hipLaunchKernelGGL((adam_fp16_vec_kernel<kAdamUnroll, false>), dim3(grid), dim3(kAdamThreads), 0, s, nvec,
+                hipLaunchKernelGGL((adam_fp16_vec_kernel<kAdamUnroll>), dim3(grid), dim3(kAdamThreads), 0, s, nvec,
                                    (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
                                    (f32x4 *)(v + head), h);
             }

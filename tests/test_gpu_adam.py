@@ -245,11 +245,13 @@ def test_one_transformer_block_flat_buffer():
 
 
 @pytest.mark.parametrize("flavour", ["bf16", "fp16"])
-@pytest.mark.parametrize("n,off", [((1 << 25) - 4096 + 3, 0), ((1 << 25) + 12345, 0), ((1 << 25) + 4096 * 3 + 1, 2)])
-def test_around_the_launch_size_where_tiles_are_handed_out_by_ticket(flavour, n, off):
-    """From 8,192 tiles on, workgroups draw their tile from a counter kept in the last vector of the 16-bit
-    output.  Whole-buffer comparison with the oracle just below and above that size, with an unaligned head:
-    every tile stepped exactly once, and the counter's place holds its real value afterwards."""
+@pytest.mark.parametrize("n,off", [((1 << 24) - 1, 0), ((1 << 24) + 2, 2), ((1 << 24) + 1024 * 7 + 5, 1), ((1 << 24) + 4 * 2048 + 3, 0),
+                                   ((1 << 25) + 12345, 0), ((1 << 25) + 4096 * 3 + 1, 2), (3 * (1 << 24) + 4 * 1537, 3)])
+def test_around_the_launch_size_where_the_resident_grid_takes_over(flavour, n, off):
+    """From 2^22 four-element groups on, a resident grid draws tiles of 256 groups from four counters kept in the
+    16-bit output (word 0 of the vectors nvec-1, nvec-513, nvec-1025, nvec-1537), whose real values a small kernel
+    restores afterwards.  Whole-buffer comparison with the oracle just below and above that size, with unaligned
+    heads and partial last tiles: every tile stepped exactly once, and the counters' places hold their real values."""
     dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
     mdt = torch.float16 if flavour == "fp16" else torch.float32
     scale = 4.0 if flavour == "fp16" else 1.0
