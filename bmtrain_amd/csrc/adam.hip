@@ -262,7 +262,6 @@ template <bool FP16>
 __global__ __launch_bounds__(kStreamThreads) void adam_stream_kernel(
     int64_t nvec, int64_t ntiles, f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, const u32x2 *__restrict__ g16,
     typename MomentVec<FP16>::type *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h) {
-    typedef typename MomentVec<FP16>::type mom_t;
     typedef StreamSet<FP16> Set;
     const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
     __shared__ uint32_t handed[2];
@@ -405,6 +404,18 @@ static hipError_t launch_split(int64_t n, bool vectorisable, int64_t head, int64
     return hipSuccess;
 }
 
+// The 16-bit parameter array is output only and hosts the tile counters of long launches: it must not share
+// memory with anything the step reads.
+static bool overlaps(const void *a, int64_t a_bytes, const void *b, int64_t b_bytes) {
+    const uintptr_t a0 = (uintptr_t)a, b0 = (uintptr_t)b;
+    return a0 < b0 + (uintptr_t)b_bytes && b0 < a0 + (uintptr_t)a_bytes;
+}
+static bool output16_overlaps_input(int64_t n, const void *p16, const void *p32, const void *g, const void *m, int64_t m_size,
+                                    const void *v) {
+    return overlaps(p16, 2 * n, p32, 4 * n) || overlaps(p16, 2 * n, g, 2 * n) || overlaps(p16, 2 * n, m, m_size * n) ||
+           overlaps(p16, 2 * n, v, 4 * n);
+}
+
 static hipError_t launch_bf16(int64_t n, float *p32, uint16_t *p16, const uint16_t *g, float *m, float *v,
                               const AdamHyper &h, hipStream_t s) {
     uintptr_t a32[3] = {(uintptr_t)p32, (uintptr_t)m, (uintptr_t)v};
@@ -488,7 +499,8 @@ struct AdamBatch {
 template <bool FP16, bool TICKET>
 __global__ __launch_bounds__(kAdamThreads) void adam_multi_kernel(AdamBatch batch, AdamHyper h, uint32_t *counter) {
     const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
-    const uint32_t tile = (uint32_t)adam_tile_index<TICKET>(counter);
+    // the tile is the same for every lane; saying so keeps the table look-ups below on the scalar unit
+    const uint32_t tile = __builtin_amdgcn_readfirstlane((uint32_t)adam_tile_index<TICKET>(counter));
     int t = 0;
     while (t + 1 < batch.count && tile >= batch.first_tile[t + 1]) t++;
     const int64_t n = batch.n[t];
@@ -567,6 +579,8 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
         const bmt_adam_tensor &t = tensors[k];
         if (t.n <= 0) continue;
         if (!t.param_fp32 || !t.param_16 || !t.grad_16 || !t.m || !t.v) return fail(-1, "adam multi launcher: null pointer");
+        if (output16_overlaps_input(t.n, t.param_16, t.param_fp32, t.grad_16, t.m, FP16 ? 2 : 4, t.v))
+            return fail(-1, "adam multi launcher: param_16 overlaps an input array");
         const bool aligned = (((uintptr_t)t.param_fp32 | (uintptr_t)t.v | (FP16 ? 0 : (uintptr_t)t.m)) & 15u) == 0 &&
                              (((uintptr_t)t.param_16 | (uintptr_t)t.grad_16 | (FP16 ? (uintptr_t)t.m : 0)) & 7u) == 0;
         const int64_t tiles = multi_tiles(t.n);
@@ -602,6 +616,8 @@ extern "C" int adam_bf16_launcher(int64_t n, void *param_fp32, void *param_bf16,
                                   float weight_decay, float bias_correction1, float bias_correction2, void *stream) {
     if (n <= 0) return 0;  // adam_cuda.cu:118
     if (!param_fp32 || !param_bf16 || !g_bf16 || !m_fp32 || !v_fp32) return fail(-1, "adam_bf16_launcher: null pointer");
+    if (output16_overlaps_input(n, param_bf16, param_fp32, g_bf16, m_fp32, 4, v_fp32))
+        return fail(-1, "adam_bf16_launcher: param_bf16 overlaps an input array");
     AdamHyper h{beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2};
     hipError_t e = launch_bf16(n, (float *)param_fp32, (uint16_t *)param_bf16, (const uint16_t *)g_bf16, (float *)m_fp32,
                                (float *)v_fp32, h, (hipStream_t)stream);
@@ -613,6 +629,8 @@ extern "C" int adam_fp16_launcher(int64_t n, void *param_fp32, void *param_fp16,
                                   float weight_decay, float bias_correction1, float bias_correction2, void *stream) {
     if (n <= 0) return 0;  // adam_cuda.cu:91
     if (!param_fp32 || !param_fp16 || !g_fp16 || !m_fp16 || !v_fp32) return fail(-1, "adam_fp16_launcher: null pointer");
+    if (output16_overlaps_input(n, param_fp16, param_fp32, g_fp16, m_fp16, 2, v_fp32))
+        return fail(-1, "adam_fp16_launcher: param_fp16 overlaps an input array");
     AdamHyper h{beta1, beta2, eps, lr, scale, weight_decay, bias_correction1, bias_correction2};
     hipError_t e = launch_fp16(n, (float *)param_fp32, (uint16_t *)param_fp16, (const uint16_t *)g_fp16,
                                   (uint16_t *)m_fp16, (float *)v_fp32, h, (hipStream_t)stream);

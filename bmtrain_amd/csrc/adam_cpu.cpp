@@ -31,6 +31,7 @@
 #include <cmath>
 #include <atomic>
 #include <condition_variable>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <mutex>
@@ -292,7 +293,13 @@ private:
     std::mutex mu_;
     std::condition_variable wake_, done_;
     const std::function<void(int)> *job_ = nullptr;
-    static constexpr int kSpinPolls = 200000;   // roughly a millisecond
+    // Roughly a millisecond of polling before a thread goes to sleep.  It buys back-to-back calls a start on all
+    // cores at once; under a CPU quota smaller than the affinity mask it costs that millisecond per call
+    // (BMT_HOST_ADAM_SPIN=0 in the environment turns the polling off).
+    static inline const int kSpinPolls = [] {
+        const char *e = getenv("BMT_HOST_ADAM_SPIN");
+        return e ? atoi(e) : 200000;
+    }();
     std::atomic<uint64_t> generation_{0};
     std::atomic<int> pending_{0};
     bool stop_ = false;
@@ -304,10 +311,10 @@ void forget_pool_in_child() { g_pool = nullptr; new (&g_pool_mutex) std::mutex()
 
 // Runs body(lo, hi, slot) over [0, n) split into `threads` contiguous chunks of
 // ceil(n / threads) elements (threads = CPUs in the caller's affinity mask, adam_cpu.hpp:54-58);
-// slot t is private to chunk t.
+// slot t is private to chunk t.  The caller reads the thread count (once per call: the mask can change under
+// a running process) and sizes whatever it indexes by slot from the same value.
 template <typename Body>
-void fan_out(int64_t n, const Body &body) {
-    const int64_t threads = affinity_cpus();
+void fan_out(int64_t n, int64_t threads, const Body &body) {
     const int64_t chunk = std::max<int64_t>((n + threads - 1) / threads, 1);
     if (threads == 1) { body(0, n, 0); return; }
     std::lock_guard<std::mutex> lock(g_pool_mutex);
@@ -329,8 +336,9 @@ using ChunkFn = void (*)(int64_t, int64_t, float *, uint16_t *, const uint16_t *
 int run(ChunkFn fn, int64_t n, void *p32, void *p16, void *delta_info, const void *g16, void *m, void *v, const Hyper &h) {
     if (n <= 0) return 0;
     if (!p32 || !p16 || !g16 || !m || !v) return bmt::fail_message(-1, "adam_cpu launcher: null pointer");
-    std::vector<Delta> parts((size_t)affinity_cpus());
-    fan_out(n, [&](int64_t lo, int64_t hi, int slot) {
+    const int64_t threads = affinity_cpus();
+    std::vector<Delta> parts((size_t)threads);
+    fan_out(n, threads, [&](int64_t lo, int64_t hi, int slot) {
         fn(lo, hi, (float *)p32, (uint16_t *)p16, (const uint16_t *)g16, (float *)m, (float *)v, h,
            delta_info ? &parts[(size_t)slot] : nullptr);
     });
@@ -370,7 +378,7 @@ extern "C" int to_fp16_from_fp32(int64_t n, const void *param_fp32, void *param_
     if (!param_fp32 || !param_fp16) return bmt::fail_message(-1, "to_fp16_from_fp32: null pointer");
     const float *src = (const float *)param_fp32;
     uint16_t *dst = (uint16_t *)param_fp16;
-    fan_out(n, [=](int64_t lo, int64_t hi, int) { for (int64_t i = lo; i < hi; i++) dst[i] = float_to_half(src[i]); });
+    fan_out(n, affinity_cpus(), [=](int64_t lo, int64_t hi, int) { for (int64_t i = lo; i < hi; i++) dst[i] = float_to_half(src[i]); });
     return 0;
 }
 
@@ -379,6 +387,6 @@ extern "C" int to_bf16_from_fp32(int64_t n, const void *param_fp32, void *param_
     if (!param_fp32 || !param_bf16) return bmt::fail_message(-1, "to_bf16_from_fp32: null pointer");
     const float *src = (const float *)param_fp32;
     uint16_t *dst = (uint16_t *)param_bf16;
-    fan_out(n, [=](int64_t lo, int64_t hi, int) { for (int64_t i = lo; i < hi; i++) dst[i] = float_to_bf16_trunc(src[i]); });
+    fan_out(n, affinity_cpus(), [=](int64_t lo, int64_t hi, int) { for (int64_t i = lo; i < hi; i++) dst[i] = float_to_bf16_trunc(src[i]); });
     return 0;
 }

@@ -57,12 +57,19 @@ class OptimManager:
 
     def __init__(self, loss_scale: Optional[float] = None, loss_scale_factor: float = 2,
                  loss_scale_steps: int = 1024, min_loss_scale=1, max_loss_scale=float("inf"),
-                 grad_scale: Optional[int] = None, defer_clip: bool = False):
+                 grad_scale: Optional[int] = None, defer_clip: bool = False, reuse_overflow_verdict: bool = False):
         # defer_clip: clip_grad_norm only measures; the clipping factor is applied inside the optimizer's fused
         # step (same parameter update, bit for bit, one pass less over the gradients), and `p.grad` keeps its
-        # unclipped values.  Needs optimizers whose step() takes `grad_coef`; otherwise clipping stays eager.
+        # unclipped values.  Taken only for a call that covers every parameter of every optimizer, all of which
+        # must take `grad_coef` in step(), and that is the only call before the step; anything else clips eagerly.
         self.defer_clip = defer_clip
         self._pending_clip = None
+        # reuse_overflow_verdict: step() trusts the inf / NaN verdict that clip_grad_norm's pass over the 16-bit
+        # gradients produced, for gradients whose memory and autograd version counter are unchanged since.  Off
+        # by default: writes through `.data`, `.detach()` views or raw pointers (what collectives do) do not
+        # move the version counter, and a gradient overwritten that way between the two calls would go
+        # unchecked.  Never used while a communicator or a copy stream is registered in `config`.
+        self.reuse_overflow_verdict = reuse_overflow_verdict
         self.loss_scale_enabled = loss_scale is not None
         self.loss_scale = loss_scale if self.loss_scale_enabled else 1
         self.steps_since_last_scale = 0
@@ -73,6 +80,7 @@ class OptimManager:
         self.grad_scale = config["zero_size"] if grad_scale is None else grad_scale
         self.optimizers = []
         self.lr_schedulers = []
+        self._clip_calls = 0          # clip_grad_norm calls since the last backward / zero_grad / step
         # verdict of the overflow scan that clip_grad_norm's pass over the gradients produced on the side
         self._known_overflow = None
 
@@ -99,20 +107,30 @@ class OptimManager:
 
     def backward(self, loss: torch.Tensor):
         self._known_overflow = None
+        if self._pending_clip is not None:      # gradients are about to be accumulated into: clip them first
+            self._scale_grads(self._pending_clip[1], self._pending_clip[0])
         self._pending_clip = None
+        self._clip_calls = 0
         self.scale_loss(loss).backward()
         self._join_load_stream(after_step=False)
 
     def zero_grad(self):
         self._known_overflow = None
         self._pending_clip = None
+        self._clip_calls = 0
         for optimizer in self.optimizers:
             optimizer.zero_grad(set_to_none=False)
 
+    def _verdict_usable(self):
+        if not self.reuse_overflow_verdict or config.get("comm") is not None or config.get("load_stream") is not None:
+            return None
+        return self._known_overflow
+
     def _overflowed(self) -> bool:
+        known = self._verdict_usable()
         for optimizer in self.optimizers:
             try:
-                check_overflow(optimizer.param_groups, self._known_overflow)
+                check_overflow(optimizer.param_groups, known)
             except OverflowError:
                 self._known_overflow = None
                 return True
@@ -130,7 +148,9 @@ class OptimManager:
                     self._justify_scale(lowered)
                 self.zero_grad()
             return
-        pending, self._pending_clip = self._pending_clip, None
+        pending = None if self._pending_clip is None else self._pending_clip[0]
+        self._pending_clip = None
+        self._clip_calls = 0
         for optimizer, lr_scheduler in zip(self.optimizers, self.lr_schedulers):
             if pending is not None:
                 optimizer.step(scale=self.loss_scale, grad_coef=pending)
@@ -148,21 +168,55 @@ class OptimManager:
                 self._justify_scale(self.loss_scale * self.loss_scale_factor)
         self._join_load_stream(after_step=True)
 
+    def _can_defer(self, parameters) -> bool:
+        """Deferred clipping hands ONE factor to every optimizer's step, which is the eager result only when
+        this call saw every parameter of every optimizer and no other call precedes the step."""
+        if not (self.defer_clip and self.optimizers and self._clip_calls == 1
+                and all(getattr(o, "supports_grad_coef", False) for o in self.optimizers)):
+            return False
+        owned = {id(p) for o in self.optimizers for group in o.param_groups for p in group["params"]}
+        return owned == {id(p) for p in parameters}
+
+    @staticmethod
+    def _scale_grads(parameters, clip_coef):
+        """`p.grad.mul_(clip_coef)` for every parameter (optim_manager.py:196-199).  Back-to-back gradients
+        are scaled by one launch.  The factor is handed over as a Python number equal to what the tensor form
+        uses on the GPU — the 0-dim fp32 tensor rounded to the gradient's dtype — which takes torch's
+        vectorised scalar kernel: same bits, 3x faster."""
+        as_number = {}
+        for g in flat_runs([p.grad.data for p in parameters if p.grad is not None]):
+            if g.is_cuda and g.dtype in (torch.float16, torch.bfloat16, torch.float32):
+                if g.dtype not in as_number:
+                    as_number[g.dtype] = float(clip_coef.to(g.dtype))
+                g.mul_(as_number[g.dtype])
+            else:
+                g.mul_(clip_coef)
+
     def clip_grad_norm(self, param_groups, max_norm, norm_type=2, eps=1e-6):
         """Clips the (still loss-scaled) gradients to ``max_norm`` in place and returns the
         unscaled total norm (optim_manager.py:158-200)."""
         scale = self.loss_scale
         scanned = None
+        if self._pending_clip is not None:
+            # a second call before the step: the first call's factor has to be in the gradients by now
+            self._scale_grads(self._pending_clip[1], self._pending_clip[0])
+            self._pending_clip = None
+            self._clip_calls = 2
+        else:
+            self._clip_calls = getattr(self, "_clip_calls", 0) + 1
         parameters = [p for group in param_groups for p in group["params"]]
-        grads = [p.grad.data if p.grad is not None else torch.zeros_like(p.data) for p in parameters]
+        # parameters without a gradient count as zeros (optim_manager.py:176-181): they add nothing
+        with_grad = [p for p in parameters if p.grad is not None]
+        grads = [p.grad.data for p in with_grad]
+        device = grads[0].device if grads else (parameters[0].device if parameters else "cuda")
         if norm_type == "inf":
-            total_norm = max(g.abs().max() for g in grads).detach()
+            total_norm = max(g.abs().max() for g in grads).detach() if grads else torch.zeros((), device=device)
         else:
             norm_type = float(norm_type)
-            device = grads[0].device if grads else "cuda"
             acc = torch.zeros(1, dtype=torch.float32, device=device)
             fused = [g for g in grads if norm_type == 2.0 and g.is_cuda and g.is_contiguous()
                      and g.dtype in (torch.float16, torch.bfloat16)]
+            fused_ids = {id(g) for g in fused}
             if fused:
                 # 16-bit gradients: one read of each tensor instead of an fp32 copy plus a norm
                 sumsq = torch.zeros(1, dtype=torch.float64, device=device)
@@ -170,30 +224,17 @@ class OptimManager:
                 for g in flat_runs(fused):
                     grad_stats(g, sumsq, flag)
                 acc += sumsq.float()
-                fused_ids = {id(g) for g in fused}
-                scanned = (flag, [p.grad for p, g in zip(parameters, grads) if id(g) in fused_ids])
-            fused_ids = {id(g) for g in fused}
+                scanned = (flag, [p.grad for p, g in zip(with_grad, grads) if id(g) in fused_ids])
             for g in grads:
                 if id(g) not in fused_ids:
                     acc += g.float().norm(norm_type) ** norm_type
             total_norm = acc[0] ** (1.0 / norm_type)
         clip_coef = float(max_norm * scale) / (total_norm + eps)
-        self._pending_clip = None
         if clip_coef < 1:
-            if self.defer_clip and self.optimizers and all(getattr(o, "supports_grad_coef", False) for o in self.optimizers):
-                self._pending_clip = clip_coef          # applied by the next step()
+            if self._can_defer(parameters):
+                self._pending_clip = (clip_coef, with_grad)          # applied by the next step()
             else:
-                # Back-to-back gradients are scaled by one launch.  The factor is handed over as a Python
-                # number equal to what `g.mul_(clip_coef)` uses on the GPU — the 0-dim fp32 tensor rounded to
-                # the gradient's dtype — which takes torch's vectorised scalar kernel: same bits, 3x faster.
-                as_number = {}
-                for g in flat_runs([p.grad.data for p in parameters if p.grad is not None]):
-                    if g.is_cuda and g.dtype in (torch.float16, torch.bfloat16, torch.float32):
-                        if g.dtype not in as_number:
-                            as_number[g.dtype] = float(clip_coef.to(g.dtype))
-                        g.mul_(as_number[g.dtype])
-                    else:
-                        g.mul_(clip_coef)
+                self._scale_grads(with_grad, clip_coef)
         # The pass over the 16-bit gradients also looked for inf / NaN, and the scaling above cannot change that
         # verdict (it multiplies by a finite factor below one, or by zero when the norm itself is infinite);
         # step() reuses it for gradients that nobody has written to since.

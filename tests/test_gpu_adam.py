@@ -196,6 +196,14 @@ def test_argument_checks():
         F.adam_bf16(p.cpu(), h, g, m, v, *a)
     with pytest.raises(AssertionError, match="float16"):
         F.adam_fp16(p, h, g, m.half(), v, *a)
+    # the 16-bit parameter is output only (long launches keep their tile counters there): a launch whose
+    # 16-bit output shares memory with the gradient or the state is refused
+    both = torch.zeros(2 * n, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="overlaps"):
+        F.adam_bf16(p, both[4:4 + n], both[:n], m, v, *a)
+    with pytest.raises(RuntimeError, match="overlaps"):
+        F.adam_bf16(p, p.view(torch.bfloat16)[:n], g, m, v, *a)
+    F.adam_bf16(p, both[n:], both[:n], m, v, *a)          # adjacent is fine
 
 
 def _fill_(x, std, gen, absolute=False, chunk=1 << 27):

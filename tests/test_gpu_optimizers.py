@@ -216,8 +216,8 @@ def test_overflow_check_and_grad_norm_over_flat_gradient_storage():
 
 
 def test_step_reuses_the_overflow_verdict_of_the_clipping_pass(monkeypatch):
-    """clip_grad_norm reads the 16-bit gradients once for norm and overflow flag; step() does not scan gradients
-    nobody has written to since, and does scan again after any in-place write."""
+    """reuse_overflow_verdict=True: clip_grad_norm reads the 16-bit gradients once for norm and overflow flag;
+    step() does not scan gradients nobody has written to since, and does scan again after an in-place write."""
     import bmtrain_amd.optim.optim_manager as om
     calls = []
     real = om.has_inf_nan
@@ -225,7 +225,7 @@ def test_step_reuses_the_overflow_verdict_of_the_clipping_pass(monkeypatch):
     torch.manual_seed(8)
     ps = [torch.nn.Parameter(torch.randn(s, device="cuda").bfloat16()) for s in (5000, 77, 4096)]
     opt = bmt.optim.AdamOptimizer(ps, lr=1e-3)
-    manager = bmt.optim.OptimManager(loss_scale=64, loss_scale_steps=1000)
+    manager = bmt.optim.OptimManager(loss_scale=64, loss_scale_steps=1000, reuse_overflow_verdict=True)
     manager.add_optimizer(opt)
 
     def grads():
@@ -254,6 +254,112 @@ def test_step_reuses_the_overflow_verdict_of_the_clipping_pass(monkeypatch):
     ps[2].grad[5] = float("inf")
     manager.step()
     assert len(calls) == 3 and manager.loss_scale == 16
+
+
+def test_overflow_is_scanned_again_by_default_and_whenever_a_runtime_is_registered(monkeypatch):
+    """A write through `.data` does not move autograd's version counter, which is how collectives and BMTrain's own
+    code touch gradients.  By default step() therefore scans every gradient itself, whatever clip_grad_norm saw;
+    with reuse switched on, a registered communicator or copy stream switches it off again."""
+    import bmtrain_amd.optim.optim_manager as om
+    torch.manual_seed(18)
+    ps = [torch.nn.Parameter(torch.randn(s, device="cuda").bfloat16()) for s in (3000, 500)]
+    opt = bmt.optim.AdamOptimizer(ps, lr=1e-3)
+
+    def grads():
+        for p in ps:
+            p.grad = (torch.randn_like(p.float()) * 64).bfloat16()
+
+    manager = bmt.optim.OptimManager(loss_scale=64, loss_scale_steps=1000)        # default: no reuse
+    manager.add_optimizer(opt)
+    grads()
+    manager.clip_grad_norm(opt.param_groups, max_norm=1e9)
+    version = ps[0].grad._version
+    ps[0].grad.data[7] = float("inf")                                   # raw write: same version counter
+    assert ps[0].grad._version == version
+    manager.step()
+    assert manager.loss_scale == 32 and "step" not in opt.state.get(ps[0], {})      # seen, step skipped
+
+    trusting = bmt.optim.OptimManager(loss_scale=64, loss_scale_steps=1000, reuse_overflow_verdict=True)
+    trusting.add_optimizer(opt)
+    monkeypatch.setitem(om.config, "comm", object())                    # a distributed runtime is present
+    grads()
+    trusting.clip_grad_norm(opt.param_groups, max_norm=1e9)
+    ps[1].grad.data[3] = float("nan")
+    trusting.step()
+    assert trusting.loss_scale == 32
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_clip_grad_norm_with_a_parameter_that_has_no_gradient(dtype):
+    """Frozen or unused parameters have `grad is None`; they count as zeros for the norm (optim_manager.py:176-181)
+    and are passed over by clipping, overflow check and step."""
+    torch.manual_seed(19)
+    ps = [torch.nn.Parameter((torch.randn(s, device="cuda") * 0.02).to(dtype)) for s in (4096, 300, 1000)]
+    opt = bmt.optim.AdamOptimizer(ps, lr=1e-3)
+    for reuse in (False, True):
+        manager = bmt.optim.OptimManager(loss_scale=8, reuse_overflow_verdict=reuse)
+        manager.add_optimizer(opt)
+        ps[0].grad = (torch.randn(4096, device="cuda") * 8).to(dtype)
+        ps[1].grad = None
+        ps[2].grad = (torch.randn(1000, device="cuda") * 8).to(dtype)
+        want = torch.sqrt(ps[0].grad.float().norm() ** 2 + ps[2].grad.float().norm() ** 2) / 8
+        got = manager.clip_grad_norm(opt.param_groups, max_norm=0.1)
+        assert abs(got.item() - want.item()) <= 1e-5 * want.item()
+        before = ps[1].detach().clone()
+        manager.step()
+        assert torch.equal(ps[1].detach(), before) and len(opt.state[ps[1]]) == 0
+    assert opt.state[ps[0]]["step"] == 2
+    none_at_all = [torch.nn.Parameter(torch.zeros(10, device="cuda", dtype=dtype))]
+    manager = bmt.optim.OptimManager(loss_scale=8)
+    assert manager.clip_grad_norm([{"params": none_at_all}], max_norm=1.0).item() == 0.0
+    assert manager.clip_grad_norm([{"params": none_at_all}], max_norm=1.0, norm_type="inf").item() == 0.0
+
+
+def test_deferred_clipping_is_taken_only_when_one_call_covers_everything():
+    """Two optimizers clipped separately (each call with its own max_norm), a subset of the parameters, two calls in
+    a row, a backward pass between clipping and step: in all of these one deferred factor for every optimizer would
+    be wrong, so the manager clips eagerly and the result equals that of a manager without defer_clip, bit for bit."""
+    dtype = torch.bfloat16
+
+    def build(defer):
+        torch.manual_seed(21)
+        a = [torch.nn.Parameter((torch.randn(s, device="cuda") * 0.02).to(dtype)) for s in (5000, 128)]
+        b = [torch.nn.Parameter((torch.randn(s, device="cuda") * 0.02).to(dtype)) for s in (2048, 77)]
+        oa, ob = bmt.optim.AdamOptimizer(a, lr=1e-3), bmt.optim.AdamOptimizer(b, lr=2e-3, weight_decay=0.01)
+        man = bmt.optim.OptimManager(loss_scale=16, defer_clip=defer)
+        man.add_optimizer(oa); man.add_optimizer(ob)
+        return a, b, oa, ob, man
+
+    def same(x, y):
+        return all(torch.equal(p.detach().view(torch.int16), q.detach().view(torch.int16)) for p, q in zip(x, y))
+
+    ea, eb, eoa, eob, eman = build(False)
+    da, db, doa, dob, dman = build(True)
+    scenarios = ["per optimizer", "subset", "twice", "all at once"]
+    for step, scenario in enumerate(scenarios):
+        torch.manual_seed(100 + step)
+        for p, q in zip(ea + eb, da + db):
+            g = (torch.randn(p.numel(), device="cuda") * 16).to(dtype)
+            p.grad, q.grad = g.clone(), g.clone()
+        for man, oa, ob, a in ((eman, eoa, eob, ea), (dman, doa, dob, da)):
+            if scenario == "per optimizer":
+                man.clip_grad_norm(oa.param_groups, max_norm=0.3)
+                man.clip_grad_norm(ob.param_groups, max_norm=0.05)
+            elif scenario == "subset":
+                man.clip_grad_norm([{"params": a[:1]}], max_norm=0.2)
+            elif scenario == "twice":
+                man.clip_grad_norm(oa.param_groups + ob.param_groups, max_norm=0.5)
+                man.clip_grad_norm(oa.param_groups + ob.param_groups, max_norm=0.1)
+            else:
+                man.clip_grad_norm(oa.param_groups + ob.param_groups, max_norm=0.4)
+        if scenario == "all at once":          # the one case that is deferred: gradients untouched, same update
+            assert dman._pending_clip is not None and not same([p.grad for p in ea], [q.grad for q in da])
+        else:
+            assert dman._pending_clip is None and same([p.grad for p in ea + eb], [q.grad for q in da + db]), scenario
+        eman.step(); dman.step()
+        assert same(ea + eb, da + db), scenario
+        for p, q in zip(ea, da):
+            assert torch.equal(eoa.state[p]["exp_avg_sq"], doa.state[q]["exp_avg_sq"]), scenario
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
