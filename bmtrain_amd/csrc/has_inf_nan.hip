@@ -11,6 +11,7 @@
 // that saw a hit issues a relaxed atomic byte store out[0] = 1 (after a look at the
 // flag: once it is up nobody stores again).  When nothing is found the kernel writes
 // nothing, which keeps the flag sticky across calls.
+#include <atomic>
 #include "bmt_device.h"
 #include "bmt_host.h"
 #include "../../include/bmt_hip.h"
@@ -196,7 +197,39 @@ static int grad_stats(int64_t n, const void *g, void *sumsq, void *flag, void *w
     return e == hipSuccess ? 0 : fail((int)e, who, e);
 }
 
+// ---- the same pass for callers that cannot allocate -------------------------------------------
+// The partial sums go to a fixed array in device memory instead of a caller's workspace.  Every GPU the
+// library runs on holds its own copy of the array at its own address; the address is looked up once per
+// device (with that device current) and used from then on — the array's name is only a host-side handle.
+constexpr int64_t kStaticPartials = (int64_t)1 << 20;                     // 4 MiB: gradients of up to 2^36 elements
+static __device__ __align__(256) float stats_scratch[kStaticPartials];
+static std::atomic<float *> stats_scratch_ptr[64];                         // per device, null until looked up
+
+static float *static_partials(const char **why) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= 64) { *why = "grad_stats_noalloc_launcher: no current device"; return nullptr; }
+    float *ptr = stats_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(stats_scratch));
+        if (e != hipSuccess || ptr == nullptr) { *why = "grad_stats_noalloc_launcher: hipGetSymbolAddress failed"; return nullptr; }
+        stats_scratch_ptr[dev].store(ptr, std::memory_order_release);     // every thread finds the same address
+    }
+    return ptr;
+}
+
 }  // namespace bmt
+
+extern "C" int grad_stats_noalloc_launcher(int64_t n, const void *g_16, int32_t is_bf16, void *sumsq, void *flag, void *stream) {
+    if (n <= 0) return 0;
+    if (bmt::stats_tiles(n, g_16, nullptr, nullptr) > bmt::kStaticPartials)
+        return bmt::fail(-1, "grad_stats_noalloc_launcher: more than 2^36 elements; use grad_stats_*_launcher with a workspace");
+    const char *why = "";
+    float *partials = bmt::static_partials(&why);
+    if (partials == nullptr) return bmt::fail(-1, why);
+    return is_bf16 ? bmt::grad_stats<bmt::BFloat16>(n, g_16, sumsq, flag, partials, stream, "grad_stats_noalloc_launcher")
+                   : bmt::grad_stats<bmt::Half>(n, g_16, sumsq, flag, partials, stream, "grad_stats_noalloc_launcher");
+}
 
 extern "C" int has_nan_inf_fp16_launcher(int64_t n, const void *g_fp16, void *mid, void *out, void *stream) {
     (void)mid;

@@ -197,6 +197,18 @@ BMT_API int grad_stats_fp16_launcher(int64_t n, const void *g_fp16, void *sumsq,
 BMT_API int grad_stats_bf16_launcher(int64_t n, const void *g_bf16, void *sumsq, void *flag, void *workspace,
                              void *stream);
 
+/*
+ * grad_stats_noalloc_launcher — no counterpart in the reference.  For callers that cannot allocate device
+ * memory (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc): the pass of
+ * grad_stats_{fp16,bf16}_launcher with its partial sums kept in a fixed 4 MiB array inside the library's own
+ * device image instead of a caller's workspace, so the call allocates nothing.  is_bf16: 0 = fp16 gradients,
+ * otherwise bf16.  Same results as the workspace form, bit for bit.  n above 2^36 elements is refused (-1).
+ * Every call on one GPU uses that GPU's one array: calls that overlap in time on the same GPU (two streams, two
+ * threads) race on it; calls that follow each other on one stream do not.
+ */
+BMT_API int grad_stats_noalloc_launcher(int64_t n, const void *g_16, int32_t is_bf16, void *sumsq, void *flag,
+                                        void *stream);
+
 #ifdef __cplusplus
 }
 #endif
