@@ -36,21 +36,28 @@ template <> __device__ __forceinline__ uint32_t neg_inf2<BFloat16>() { return 0x
 __device__ __forceinline__ float add_tiny(float s) { return (float)((double)s + 1e-10); }  // cross_entropy.cu:28
 
 // ---- exponentials and the quotient -------------------------------------------------
-// All exponentials here are e^(x - M) with x <= M.  They are produced multiplied by 2^64
+// All exponentials here are e^(x - M) with x <= M.  They are produced multiplied by 2^16
 // ("biased"): v_exp_f32 returns 0 for results below 2^-126, and the bias keeps everything that
-// can still matter after the division (down to 2^-190) in the normal range; the factor is
-// removed again, exactly, by the reciprocal used for the quotient.
+// can still matter after the division in the normal range — the smallest quotient a 16-bit
+// output can hold is 2^-134 (half the least bf16 subnormal), and with a divisor of at least 1 its
+// exponential is at least 2^-134, biased 2^-118.  The factor is removed again, exactly, by the
+// reciprocal used for the quotient.
 //
 // The forward kernels are close to ALU-bound (a v_exp_f32 costs four issue slots and every
 // element needs one or two), so the exponential is three instructions and the quotient one.
-// Errors stay far below half an ulp of the 16-bit result: about 2^-20 relative from rounding
-// (x - M) * log2(e) + 64 once, 2^-22 from v_exp_f32, 2^-23 from the reciprocal and the product.
+// Errors stay far below half an ulp of the 16-bit result.  The largest is the one rounding of
+// (x - M) * log2(e) + 16, half an ulp of a number between -16 and 16, i.e. 2^-21 to 2^-23 for most
+// elements (which is why the bias is no larger than it has to be: with 64 in its place that
+// rounding alone was 2^-19, and the stored softmax differed from a libm-based evaluation on 1.4 to
+// 1.8 elements in 10,000; now 0.3 to 0.4); then 2^-22 from v_exp_f32, 2^-23 from the reciprocal and
+// the product.
 constexpr float kLog2e = 1.44269502162933349609375f;       // fp32 nearest to log2(e)
-constexpr float kBias = 64.0f;
-constexpr float kTwoPowMinusBias = 5.42101086242752217e-20f;  // 2^-64
+constexpr int kBiasLog2 = 16;
+constexpr float kBias = (float)kBiasLog2;
+constexpr float kTwoPowMinusBias = 1.0f / (float)(1 << kBiasLog2);   // 2^-16, exact
 
-// 2^64 * e^(x - M).  The difference is formed first (folding M into the constant would save an
-// instruction, but rounds 64 - M * log2(e) to an error that grows with |M| and overflows for huge
+// 2^16 * e^(x - M).  The difference is formed first (folding M into the constant would save an
+// instruction, but rounds 16 - M * log2(e) to an error that grows with |M| and overflows for huge
 // M); x = -inf gives 0, NaN gives NaN.
 __device__ __forceinline__ float exp_biased(float x, float M) {
     return __builtin_amdgcn_exp2f(__builtin_fmaf(x - M, kLog2e, kBias));
@@ -58,15 +65,15 @@ __device__ __forceinline__ float exp_biased(float x, float M) {
 // The row's divisor in the two forms the kernels need.
 struct RowSum {
     float S;      // sum of exponentials + 1e-10, unbiased (for the loss)
-    float r64;    // 2^-64 / S: multiplying a biased exponential by it gives the softmax value
+    float scaled_reciprocal;    // 2^-16 / S: multiplying a biased exponential by it gives the softmax value
 };
 __device__ __forceinline__ RowSum make_row_sum(float biased_sum) {
     RowSum rs;
     rs.S = add_tiny(biased_sum * kTwoPowMinusBias);
-    rs.r64 = (1.0f / rs.S) * kTwoPowMinusBias;
+    rs.scaled_reciprocal = (1.0f / rs.S) * kTwoPowMinusBias;
     return rs;
 }
-__device__ __forceinline__ float quotient(float e_biased, const RowSum &rs) { return e_biased * rs.r64; }
+__device__ __forceinline__ float quotient(float e_biased, const RowSum &rs) { return e_biased * rs.scaled_reciprocal; }
 
 // Loss of one row; an out-of-range target that is not ignore_index yields NaN instead
 // of the reference's out-of-bounds read.
@@ -326,7 +333,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
     const u32x4 pad4 = {pad, pad, pad, pad};
 
     float m = -1e6f;   // running maximum of this lane, never below the reference's clamp
-    float s = 0.f;     // sum of 2^64 * e^(x - m) over this lane's elements so far
+    float s = 0.f;     // sum of 2^16 * e^(x - m) over this lane's elements so far
     // Folds GROUP vectors into (m, s).
     auto absorb = [&](const u32x4 (&v)[GROUP], int c0) {
         if (c0 * THREADS + (tid & ~(kWave - 1)) >= nvec) return;   // this wave is past the end of the row
@@ -459,9 +466,9 @@ constexpr int kFlatScalarThreads = 256;
 template <typename T, int OP>
 __device__ __forceinline__ float flat_elem(float s, bool is_target, float a, float b) {
     if (OP == 0) return is_target ? (s - 1.f) * a : s * a;  // a = grad_output[r]
-    return exp_biased(s, a) * b;                            // a = max, b = 2^-64 / sum
+    return exp_biased(s, a) * b;                            // a = max, b = 2^-16 / sum
 }
-// Second per-row scalar of the flat kernels: nothing for the backward, 2^-64 / sum for the softmax.
+// Second per-row scalar of the flat kernels: nothing for the backward, 2^-16 / sum for the softmax.
 template <int OP>
 __device__ __forceinline__ float flat_row_b(const float *row_b, int64_t row) {
     return OP == 1 ? kTwoPowMinusBias / row_b[row] : 0.f;
@@ -555,7 +562,7 @@ __global__ __launch_bounds__(kFlatScalarThreads) void ce_flat_scalar_kernel(
 
 // ---- row sum of exponentials given the row maximum ---------------------------------
 // One workgroup of THREADS lanes per row, two vectors per lane in flight.  The exponentials are the
-// biased ones of the forward kernels; the factor 2^64 is taken out of the sum at the end.
+// biased ones of the forward kernels; the factor 2^16 is taken out of the sum at the end.
 template <typename T, int THREADS>
 __global__ __launch_bounds__(THREADS) void sumexp_kernel(int32_t n, const uint16_t *__restrict__ x,
                                                          const float *__restrict__ row_max,

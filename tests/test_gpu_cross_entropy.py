@@ -49,7 +49,9 @@ def test_forward_against_oracle(name, dtype, n):
     softmax, loss = _forward_gpu(x, t)
     want_soft, want_loss = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
     assert ulp_distance16(bits16(softmax), want_soft).max() <= 1
-    assert (bits16(softmax) != want_soft).mean() < 0.01
+    # rarely off by its one ulp: more often for fp16 values in the normal range, whose ulp is 2^-11 of the value,
+    # than for bf16 (2^-8) or the subnormal fp16 values of long rows; the benchmark shapes have a test of their own
+    assert (bits16(softmax) != want_soft).sum() <= 3 + (1e-3 if name == "fp16" else 2e-4) * m * n
     np.testing.assert_allclose(loss.cpu().numpy(), want_loss, rtol=2e-6, atol=2e-6)
     ref32 = torch.nn.functional.cross_entropy(x.float(), t.long(), ignore_index=-100, reduction="none").numpy()
     np.testing.assert_allclose(loss.cpu().numpy(), ref32, rtol=1e-3, atol=1e-6)
@@ -300,16 +302,27 @@ def test_vocab_parallel_loss_with_one_rank(dtype):
     assert ((grad_v.float() - grad_f.float()).abs() <= ulp * grad_f.float().abs() + 1e-3).all()
 
 
-@pytest.mark.parametrize("m,n,name,dtype", [(16384, 32000, "fp16", torch.float16), (8192, 128256, "bf16", torch.bfloat16)])
-def test_language_model_head_shape(m, n, name, dtype):
-    """16,384 rows x 32,000 classes fp16 and 8,192 rows x 128,256 classes bf16, 10 % ignored, mean
-    reduction.  Seeded rows are checked against the oracle; all rows are checked through row sums, the
-    loss against torch in fp32 on the GPU, and sign / zero structure of the gradient."""
-    gen = torch.Generator(device="cuda").manual_seed(3)
-    x = (torch.randn(m, n, generator=gen, device="cuda") * 2).to(dtype)
+LM_HEADS = [(16384, 32000, "fp16", torch.float16, 2.0, 10, 3), (8192, 128256, "bf16", torch.bfloat16, 3.0, 20, 4)]
+
+
+def _lm_head_case(m, n, dtype, std, every, seed):
+    """The benchmark inputs: logits ~ N(0, std) rounded to the 16-bit type, uniform targets, one row in `every`
+    ignored (seeded permutation)."""
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.empty(m, n, dtype=dtype, device="cuda")
+    for lo in range(0, m, 1024):
+        x[lo:lo + 1024] = (torch.randn(1024, n, generator=gen, device="cuda") * std).to(dtype)
     t = torch.randint(0, n, (m,), generator=gen, device="cuda", dtype=torch.int32)
-    ignored = torch.randperm(m, generator=gen, device="cuda")[: m // 10]
-    t[ignored] = -100
+    t[torch.randperm(m, generator=gen, device="cuda")[: m // every]] = -100
+    return x, t
+
+
+@pytest.mark.parametrize("m,n,name,dtype,std,every,seed", LM_HEADS)
+def test_language_model_head_shape(m, n, name, dtype, std, every, seed):
+    """16,384 rows x 32,000 classes fp16 (logits N(0,2), 10 % ignored) and 8,192 rows x 128,256 classes bf16
+    (N(0,3), 5 % ignored), mean reduction.  Seeded rows are checked against the oracle; all rows are checked
+    through row sums, the loss against torch in fp32 on the GPU, and sign / zero structure of the gradient."""
+    x, t = _lm_head_case(m, n, dtype, std, every, seed)
     softmax = torch.empty_like(x)
     out = torch.empty(m, dtype=torch.float32, device="cuda")
     F.cross_entropy_forward(m, n, x, t, softmax, out, -100)
@@ -337,6 +350,65 @@ def test_language_model_head_shape(m, n, name, dtype):
     tv = t[valid].long()
     at_target = softmax[valid].gather(1, tv[:, None])
     assert (at_target < 0).all()
+    del x, softmax
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("m,n,name,dtype,std,every,seed", LM_HEADS)
+def test_gradient_parity_at_the_benchmark_shapes(m, n, name, dtype, std, every, seed, capsys):
+    """How far the two kernels are from the oracle's chain (libm expf, IEEE division, two roundings to 16 bits) on
+    the benchmark inputs, in units of the types involved, at upstream scales 1, 32768 and 2^20.  The kernels run on
+    the full shape; a seeded sample of rows (24 M elements) is compared.
+
+    Stored softmax: never more than 1 ulp off, and different on fewer than 1 element in 10,000.
+    Gradient, in ulps of the gradient's own 16-bit value: identical wherever the stored softmax is; bf16: never
+    more than 1 ulp off.  fp16 at 32,000 classes: the stored softmax is mostly *subnormal* (p ~ 3e-5 < 6.1e-5), so
+    one step of it is 2^-24 whatever the value, while the gradient p * grad_output * scale is a normal number whose
+    ulp can be far smaller than 2^-24 * grad_output * scale: a softmax off by its one ulp can be several gradient
+    ulps off (the same holds between any two evaluations of the reference's expression with different expf
+    implementations).  Those elements are bounded by that one softmax step, and counted."""
+    x, t = _lm_head_case(m, n, dtype, std, every, seed)
+    sample = 768 if n == 32000 else 192
+    rows = torch.randperm(m, generator=torch.Generator().manual_seed(seed))[:sample].sort().values.cuda()
+    softmax = torch.empty_like(x)
+    out = torch.empty(m, dtype=torch.float32, device="cuda")
+    F.cross_entropy_forward(m, n, x, t, softmax, out, -100)
+    ts = t[rows].cpu().numpy()
+    want_soft, want_loss = oracle.ce_forward(bits16(x[rows]), ts, -100, name)
+    want_soft = want_soft.reshape(sample, n)
+    got_soft = bits16(softmax[rows]).reshape(sample, n)
+    dist = ulp_distance16(got_soft, want_soft)
+    report = [f"{name} {m}x{n}: stored softmax differs on {np.mean(dist != 0):.2e} of {dist.size} elements, max {dist.max()} ulp"]
+    assert dist.max() <= 1 and np.mean(dist != 0) < 1e-4
+    np.testing.assert_allclose(out[rows].cpu().numpy(), want_loss, rtol=2e-6, atol=2e-6)
+    valid = (t != -100).float()
+    for upstream in (1.0, 32768.0, 2.0 ** 20):
+        v = (valid / valid.sum() * upstream).contiguous()
+        grad = softmax.clone()
+        F.cross_entropy_backward_inplace(m, n, v, t, grad, -100)
+        got = bits16(grad[rows]).reshape(sample, n)
+        del grad
+        vs = v[rows].cpu().numpy()
+        want = np.ascontiguousarray(want_soft.copy())
+        oracle.ce_backward_inplace(vs, ts, want, -100, name)
+        same_input = np.ascontiguousarray(got_soft.copy())
+        oracle.ce_backward_inplace(vs, ts, same_input, -100, name)
+        assert np.array_equal(got, same_input)                       # the backward kernel itself is exact
+        err = np.abs(_value16(got.reshape(-1), dtype) - _value16(want.reshape(-1), dtype))
+        ulps = (err / _ulp_size16(want.reshape(-1), dtype)).reshape(sample, n)
+        assert not np.any((ulps != 0) & (dist == 0))                 # differences only where the softmax differs
+        report.append(f"  grad_output scale {upstream:g}: gradient differs on {np.mean(ulps != 0):.2e}, by more than 1 ulp on "
+                      f"{np.mean(ulps > 1):.2e}, max {ulps.max():.0f} ulp")
+        assert np.mean(ulps != 0) < 1e-4
+        if dtype == torch.bfloat16:
+            assert ulps.max() <= 1
+        else:
+            assert np.mean(ulps > 1) < 5e-5
+            step = _ulp_size16(want_soft.reshape(-1), dtype).reshape(sample, n) * np.abs(vs.astype(np.float64))[:, None]
+            bound = step + _ulp_size16(want.reshape(-1), dtype).reshape(sample, n)
+            assert np.all(err.reshape(sample, n) <= bound)
+    with capsys.disabled():
+        print("\n" + "\n".join(report))
     del x, softmax
     torch.cuda.empty_cache()
 
