@@ -115,8 +115,8 @@ def cpu_baseline():
         "elements_per_s": round(n / median, 1),
     }
     # the reference's bf16 host path (a scalar loop per thread), same inputs, 10 steps
+    gb = [(torch.randn(n, generator=gen) * 1e-3).bfloat16().view(torch.int16).numpy().view(np.uint16).copy()]
     if ref is not None:
-        gb = [(torch.randn(n, generator=gen) * 1e-3).bfloat16().view(torch.int16).numpy().view(np.uint16).copy()]
         bf_times = []
         for k in range(10):
             bc1, bc2 = oracle.bias_corrections(0.9, 0.999, k + 1)
@@ -127,6 +127,27 @@ def cpu_baseline():
         bf_times.sort()
         out["adam_bf16_GBps"] = round(ADAM_BF16_BYTES * n / bf_times[5] / 1e9, 3)
         out["adam_bf16_sample"] = f"adam_cpu bf16 grads, N=2^24, 10 steps, median {bf_times[5] * 1e3:.2f} ms/step"
+    # this repository's own host Adam (the offload optimizer's kernel) on the same inputs and cores, beside it
+    try:
+        from bmtrain_amd import C
+        prod = {}
+        for label, launcher, grad_bits, scale in (("fp16", C.adam_cpu_fp16_launcher, grads[0], 1024.0),
+                                                  ("bf16", C.adam_cpu_bf16_launcher, gb[0], 1.0)):
+            ts = []
+            for k in range(20):
+                bc1, bc2 = oracle.bias_corrections(0.9, 0.999, k + 1)
+                t0 = time.perf_counter()
+                launcher(n, p.ctypes.data, h.ctypes.data, 0, grad_bits.ctypes.data, m.ctypes.data, v.ctypes.data,
+                         0.9, 0.999, 1e-8, 1e-3, scale, 0.01, bc1, bc2)
+                ts.append(time.perf_counter() - t0)
+            ts.sort()
+            prod[label] = {"GBps_median": round(ADAM_BF16_BYTES * n / ts[len(ts) // 2] / 1e9, 1),
+                           "GBps_best": round(ADAM_BF16_BYTES * n / ts[0] / 1e9, 1),
+                           "ms_median": round(ts[len(ts) // 2] * 1e3, 3), "ms_min": round(ts[0] * 1e3, 3)}
+        out["product_host_adam"] = dict(prod, cores=cores, sample="adam_cpu_{fp16,bf16}_launcher of libbmt_hip.so, N=2^24, "
+                                        "20 steps back to back, same buffers and cores as the reference's kernel above")
+    except Exception as exc:                      # the baseline must not sink the GPU numbers
+        out["product_host_adam"] = {"error": repr(exc)}
     # CPU cross-entropy (torch), fp32 as FusedCrossEntropy itself does for fp32 input
     torch.set_num_threads(cores)
     for key, rows, classes, std, every in (("ce", 256, 128256, 3.0, 20), ("ce_32000", 1024, 32000, 2.0, 10)):
@@ -146,22 +167,38 @@ def cpu_baseline():
     return out
 
 
+def timed_batches(torch, fn, iters=20, per_batch=4):
+    """(mean, median, min) of the time per call in ms.  The calls run back to back in batches of `per_batch`, each
+    batch bracketed by one pair of events (an event between every two short launches would add its own gap to
+    each of them); mean over all batches, median and minimum over the batches."""
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    batches = max(iters // per_batch, 3)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(batches)]
+    for a, b in evs:
+        a.record()
+        for _ in range(per_batch):
+            fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) / per_batch for a, b in evs)
+    return sum(ts) / len(ts), ts[len(ts) // 2], ts[0]
+
+
 def other_workloads(torch, dev, LF, OF, iters=20):
     """The other configurations the targets are stated on (not the headline line): one transformer block's
     flat Adam step (202,383,360 elements, bf16, t = 100; also fp16 and the gradient statistics pass over the
     same gradients), the fp16 overflow scan over 2^30 elements, and the fp16 language-model head
     cross-entropy (16,384 rows x 32,000 classes, 10 % ignored)."""
     def timed(fn):
-        for _ in range(3):
-            fn()
-        torch.cuda.synchronize()
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        for _ in range(iters):
-            fn()
-        b.record()
-        torch.cuda.synchronize()
-        return a.elapsed_time(b) / iters
+        return timed_batches(torch, fn, iters)
+
+    def entry(stats, nbytes, **more):
+        mean, median, low = stats
+        gbps = nbytes / (mean * 1e-3) / 1e9
+        return dict({"ms": round(mean, 4), "ms_median": round(median, 4), "ms_min": round(low, 4),
+                     "achieved_GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}, **more)
 
     out = {}
     gen = torch.Generator(device=dev).manual_seed(1)
@@ -171,21 +208,17 @@ def other_workloads(torch, dev, LF, OF, iters=20):
     p32, mom, var = (torch.empty(n, device=dev) for _ in range(3))
     fill_normal_(p32, 0.02, gen); fill_normal_(mom, 1e-4, gen); fill_normal_(var, 1e-6, gen, absolute=True)
     fill_normal_(grad, 1e-3, gen)
-    ms = timed(lambda: OF.adam_bf16(p32, p16, grad, mom, var, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100))
-    gbps = ADAM_BF16_BYTES * n / (ms * 1e-3) / 1e9
-    out["adam_bf16_one_block_202M"] = {"ms": round(ms, 4), "achieved_GBps": round(gbps, 1),
-                                       "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+    out["adam_bf16_one_block_202M"] = entry(
+        timed(lambda: OF.adam_bf16(p32, p16, grad, mom, var, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100)), ADAM_BF16_BYTES * n,
+        buffers="five separate allocations made for this measurement")
     h16, g16, m16 = p16.view(torch.float16), grad.view(torch.float16), mom.view(torch.float16)[:n]
     g16.copy_(grad.float().mul_(1024.0)); m16.zero_(); fill_normal_(var, 1e-3, gen, absolute=True)
-    ms = timed(lambda: OF.adam_fp16(p32, h16, g16, m16, var, 0.9, 0.999, 1e-8, 1e-3, 1024.0, 0.01, 100))
-    gbps = 24 * n / (ms * 1e-3) / 1e9
-    out["adam_fp16_one_block_202M"] = {"ms": round(ms, 4), "achieved_GBps": round(gbps, 1),
-                                       "frac": round(gbps / HBM_PEAK_GBPS, 4), "bytes_per_element": 24}
+    out["adam_fp16_one_block_202M"] = entry(
+        timed(lambda: OF.adam_fp16(p32, h16, g16, m16, var, 0.9, 0.999, 1e-8, 1e-3, 1024.0, 0.01, 100)), 24 * n,
+        bytes_per_element=24)
     sumsq = torch.zeros(1, dtype=torch.float64, device=dev)
     flag = torch.zeros(1, dtype=torch.uint8, device=dev)
-    ms = timed(lambda: OF.grad_stats(grad, sumsq, flag))
-    gbps = 2 * n / (ms * 1e-3) / 1e9
-    out["grad_stats_bf16_202M"] = {"ms": round(ms, 4), "achieved_GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+    out["grad_stats_bf16_202M"] = entry(timed(lambda: OF.grad_stats(grad, sumsq, flag)), 2 * n)
     del p16, grad, p32, mom, var, h16, g16, m16
     torch.cuda.empty_cache()
 
@@ -193,9 +226,7 @@ def other_workloads(torch, dev, LF, OF, iters=20):
     g = torch.empty(n16, dtype=torch.float16, device=dev)
     fill_normal_(g, 1e-3, gen)
     flag = torch.zeros(1, dtype=torch.uint8, device=dev)[0]
-    ms = timed(lambda: LF.has_inf_nan(g, flag))
-    gbps = SCAN_BYTES * n16 / (ms * 1e-3) / 1e9
-    out["has_inf_nan_fp16_2^30"] = {"ms": round(ms, 4), "achieved_GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+    out["has_inf_nan_fp16_2^30"] = entry(timed(lambda: LF.has_inf_nan(g, flag)), SCAN_BYTES * n16)
     del g
     torch.cuda.empty_cache()
 
@@ -213,10 +244,33 @@ def other_workloads(torch, dev, LF, OF, iters=20):
     def fwd_bwd():
         LF.cross_entropy_forward(rows, classes, x, t, soft, loss, -100)
         LF.cross_entropy_backward_inplace(rows, classes, go, t, soft, -100)
-    ms = timed(fwd_bwd)
-    gbps = ce_bytes_per_row(classes) * rows / (ms * 1e-3) / 1e9
-    out["ce_fp16_16384x32000_fwd_bwd"] = {"ms": round(ms, 4), "rows_per_s": round(rows / (ms * 1e-3), 1),
-                                          "achieved_GBps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+    stats = timed(fwd_bwd)
+    out["ce_fp16_16384x32000_fwd_bwd"] = entry(stats, ce_bytes_per_row(classes) * rows, rows_per_s=round(rows / (stats[0] * 1e-3), 1))
+    out["ce_fp16_16384x32000_forward"] = entry(
+        timed(lambda: LF.cross_entropy_forward(rows, classes, x, t, soft, loss, -100)), (4 * classes + 8) * rows)
+    del x, soft
+    torch.cuda.empty_cache()
+
+    # the offload optimizer on one block: gradients device -> host, host Adam, 16-bit parameters host -> device
+    import bmtrain_amd as bmt
+    n = 202_383_360
+    param = torch.nn.Parameter(torch.zeros(n, dtype=torch.bfloat16, device=dev))
+    offload = bmt.optim.AdamOffloadOptimizer([param], lr=1e-3, weight_decay=0.01)
+    g = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    fill_normal_(g, 1e-3, gen)
+    walls = []
+    for k in range(6):
+        param.grad = g
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        offload.step()
+        torch.cuda.synchronize()
+        walls.append((time.perf_counter() - t0) * 1e3)
+    walls = sorted(walls[1:])                 # the first step allocates and pins the host state
+    out["adam_offload_step_bf16_202M"] = {
+        "ms_wall_median": round(walls[len(walls) // 2], 2), "ms_wall_min": round(walls[0], 2), "steps": len(walls),
+        "elements_per_s": round(n / (walls[len(walls) // 2] * 1e-3), 1),
+        "what": "AdamOffloadOptimizer.step(): D2H of gradients, host Adam, H2D of the 16-bit copy, pieces pipelined (PCIe both ways)"}
     return out
 
 
@@ -256,6 +310,55 @@ def tensor_list_step(torch, p16, grad, p32, mom, var, merge, batch=True, iters=5
     gbps = ADAM_BF16_BYTES * p16.numel() / (ms * 1e-3) / 1e9
     return {"tensors": len(shapes), "ms_wall": round(ms, 3), "achieved_GBps": round(gbps, 1),
             "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+
+
+def full_model_side_measurements(torch, OF, p16, grad, p32, mom, var, iters=5):
+    """On the resident 6.74 B-element state: the one-pass gradient statistics, and `clip_grad_norm` + `step()`
+    through OptimManager with clipping active — eager (the gradients are scaled in place, then stepped) and
+    deferred (the step's kernels apply the factor; one pass less over the gradients)."""
+    import bmtrain_amd as bmt
+    n = grad.numel()
+    out = {}
+    sumsq = torch.zeros(1, dtype=torch.float64, device=grad.device)
+    flag = torch.zeros(1, dtype=torch.uint8, device=grad.device)
+    OF.grad_stats(grad, sumsq, flag)
+    torch.cuda.synchronize()
+    mean, median, low = timed_batches(torch, lambda: OF.grad_stats(grad, sumsq, flag), 12)
+    out["grad_stats_bf16_6.74B"] = {"ms": round(mean, 4), "ms_median": round(median, 4), "ms_min": round(low, 4),
+                                    "achieved_GBps": round(2 * n / (mean * 1e-3) / 1e9, 1),
+                                    "frac": round(2 * n / (mean * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+    layer = [(4096, 4096)] * 4 + [(11008, 4096)] * 2 + [(4096, 11008)] + [(4096,)] * 2
+    shapes = [(32000, 4096)] + layer * 32 + [(4096,), (32000, 4096)]
+    gen = torch.Generator(device=grad.device).manual_seed(44)
+    for label, defer in (("eager", False), ("deferred", True)):
+        params, lo = [], 0
+        for shape in shapes:
+            size = 1
+            for d in shape:
+                size *= d
+            q = torch.nn.Parameter(p16[lo:lo + size].view(shape))
+            q.grad = grad[lo:lo + size].view(shape)
+            params.append((q, lo, size, shape))
+            lo += size
+        opt = bmt.optim.AdamOptimizer([q[0] for q in params], lr=1e-3, weight_decay=0.01)
+        for q, lo, size, shape in params:
+            opt.state[q] = {"step": 99, "exp_avg": mom[lo:lo + size].view(shape), "exp_avg_sq": var[lo:lo + size].view(shape),
+                            "_param_fp32": p32[lo:lo + size].view(shape)}
+        manager = bmt.optim.OptimManager(loss_scale=1.0, defer_clip=defer, loss_scale_steps=10 ** 9)
+        manager.add_optimizer(opt)
+        walls = []
+        for k in range(iters + 1):
+            fill_normal_(grad, 1e-3, gen)                 # eager clipping shrinks the gradients in place: refill
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            manager.clip_grad_norm(opt.param_groups, max_norm=1e-3)
+            manager.step()
+            torch.cuda.synchronize()
+            walls.append((time.perf_counter() - t0) * 1e3)
+        walls = sorted(walls[1:])
+        out["clip_grad_norm_plus_step_6.74B_" + label] = {"ms_wall_median": round(walls[len(walls) // 2], 3),
+                                                          "ms_wall_min": round(walls[0], 3), "steps": len(walls)}
+    return out
 
 
 def load_measured_traffic():
@@ -350,7 +453,12 @@ def main():
         softmax.copy_(logits)
         torch.cuda.synchronize()
 
-    ms = {name: sum(ev[i].elapsed_time(ev[i + 1]) for ev in all_events) / args.steps for i, name in enumerate(names)}
+    per_step = {name: sorted(ev[i].elapsed_time(ev[i + 1]) for ev in all_events) for i, name in enumerate(names)}
+    ms = {name: sum(ts) / len(ts) for name, ts in per_step.items()}
+
+    def spread(name):
+        ts = per_step[name]
+        return {"ms_median": round(ts[len(ts) // 2], 4), "ms_min": round(ts[0], 4)}
     adam_gbps = ADAM_BF16_BYTES * n / (ms["adam"] * 1e-3) / 1e9
     scan_gbps = SCAN_BYTES * n / (ms["has_inf_nan"] * 1e-3) / 1e9
     ce_ms = ms["ce_forward"] + ms["ce_backward"]
@@ -376,29 +484,44 @@ def main():
         "config": {"workload": workload, "elements": n, "ce_rows": rows, "ce_classes": classes,
                    "grad_dtype": "bf16", "adam_step": "t=100+k, lr 1e-3, betas (0.9,0.999), eps 1e-8, wd 0.01, scale 1"},
         "roofline": {
-            "kernel": "adam_bf16_vec_kernel",
+            "kernel": "adam_stream_kernel<bf16>" if n >= (1 << 24) else "adam_bf16_vec_kernel",
             "bound": "hbm",
             "achieved": round(adam_gbps, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(adam_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": traffic.get("adam_bf16_vec_kernel", {}).get("bytes_per_launch") if not args.small else None,
+            "traffic": traffic.get("adam_stream_kernel", {}).get("bytes_per_launch") if not args.small else None,
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command, read from "
+                              "profiles/hbm_traffic.json (not measured by this run)",
             "algorithmic_bytes_per_launch": ADAM_BF16_BYTES * n,
             "ms_per_launch": round(ms["adam"], 4),
+            **spread("adam"),
         },
         "ce_fwd_bwd_rows_per_s": round(ce_rows_per_s, 1),
         "other_kernels": {
-            "has_inf_nan": {"ms": round(ms["has_inf_nan"], 4), "achieved_GBps": round(scan_gbps, 1),
+            "has_inf_nan": {"ms": round(ms["has_inf_nan"], 4), **spread("has_inf_nan"), "achieved_GBps": round(scan_gbps, 1),
                             "frac": round(scan_gbps / HBM_PEAK_GBPS, 4), "algorithmic_bytes": SCAN_BYTES * n},
-            "ce_forward": {"ms": round(ms["ce_forward"], 4), "achieved_GBps": round(ce_fwd_gbps, 1),
+            "ce_forward": {"ms": round(ms["ce_forward"], 4), **spread("ce_forward"), "achieved_GBps": round(ce_fwd_gbps, 1),
                            "frac": round(ce_fwd_gbps / HBM_PEAK_GBPS, 4)},
-            "ce_backward": {"ms": round(ms["ce_backward"], 4), "achieved_GBps": round(ce_bwd_gbps, 1),
+            "ce_backward": {"ms": round(ms["ce_backward"], 4), **spread("ce_backward"), "achieved_GBps": round(ce_bwd_gbps, 1),
                             "frac": round(ce_bwd_gbps / HBM_PEAK_GBPS, 4)},
             "ce_fwd_bwd": {"ms": round(ce_ms, 4), "achieved_GBps": round(ce_gbps, 1),
                            "frac": round(ce_gbps / HBM_PEAK_GBPS, 4), "bytes_per_row": ce_bytes_per_row(classes)},
         },
     }
     side = not (args.small or args.no_other_workloads)
+    block_in_place = model_side = None
+    if side:
+        # one transformer block's worth of the resident model state (what a training process steps when it steps
+        # one block): the first 202,383,360 elements of the five 6.74 B-element arrays
+        nb = 202_383_360
+        step_block = lambda: OF.adam_bf16(p32[:nb], p16[:nb], grad[:nb], mom[:nb], var[:nb], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100)
+        mean, median, low = timed_batches(torch, step_block, 40)
+        block_in_place = {"ms": round(mean, 4), "ms_median": round(median, 4), "ms_min": round(low, 4),
+                          "achieved_GBps": round(ADAM_BF16_BYTES * nb / (mean * 1e-3) / 1e9, 1),
+                          "frac": round(ADAM_BF16_BYTES * nb / (mean * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                          "buffers": "the first block's slice of the resident 6.74 B-element state"}
+        model_side = full_model_side_measurements(torch, OF, p16, grad, p32, mom, var)
     tensor_list = None if not side else {
         "adjacent_tensors_merged": tensor_list_step(torch, p16, grad, p32, mom, var, True),
         "32_tensors_per_launch": tensor_list_step(torch, p16, grad, p32, mom, var, False),
@@ -409,6 +532,8 @@ def main():
     if side:
         result["other_workloads"] = other_workloads(torch, dev, LF, OF)
         result["other_workloads"]["adam_bf16_llama7b_291_tensors_via_optimizer_step"] = tensor_list
+        result["other_workloads"]["adam_bf16_one_block_202M_in_model_state"] = block_in_place
+        result["other_workloads"].update(model_side)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
