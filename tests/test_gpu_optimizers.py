@@ -89,6 +89,61 @@ def test_fused_and_offload_agree_closely(dtype):
         bmt.optim.AdamOptimizer.get_avg_delta()
 
 
+def _host_simd_level():
+    have = set()
+    with open("/proc/cpuinfo") as f:
+        for line in f:
+            if line.startswith("flags"):
+                have = set(line.split(":", 1)[1].split())
+                break
+    narrow = {"avx", "fma", "f16c"} <= have
+    return 2 if ("avx512f" in have and narrow) else (1 if narrow else 0)
+
+
+def test_offload_optimizer_on_the_reference_cpu_configuration():
+    """The configuration the reference's CPU path is quoted on, exactly, through AdamOffloadOptimizer on this box:
+    N = 2^24 fp32 master parameters ~ N(0, 0.02), fp16 gradients ~ N(0, 1e-3) * 1024, m = v = 0, lr 1e-3, betas
+    (0.9, 0.999), eps 1e-8, weight decay 0.01, loss scale 1024, 10 steps, fixed seed.  fp32 state on the host and the
+    fp16 copy on the device must equal, bit for bit, the oracle's restatement of adam_cpu_fp16_launcher
+    (adam_cpu.hpp:504-533) run at this host's SIMD level and thread count over the same pieces the optimizer cuts
+    the tensor into (which elements fall to the vector or the scalar tree depends on both, adam_cpu.hpp:332-351)."""
+    import os
+    import oracle
+    from conftest import bits16, f32_bits
+    n = 1 << 24
+    gen = torch.Generator().manual_seed(0)
+    master = torch.randn(n, generator=gen) * 0.02
+    param = torch.nn.Parameter(master.half().cuda())
+    opt = bmt.optim.AdamOffloadOptimizer([param], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01)
+    # the optimizer derives its fp32 master from the 16-bit parameter; the configuration states the master itself
+    with torch.no_grad():
+        opt._init_state(param)["_param_fp32"].copy_(master)
+    po, mo, vo = master.numpy().copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    ho = np.zeros(n, np.uint16)
+    threads, level = len(os.sched_getaffinity(0)), _host_simd_level()
+    piece = opt.chunk_elements
+    for step in range(1, 11):
+        g = (torch.randn(n, generator=gen) * 1e-3 * 1024).half()
+        param.grad = g.cuda()
+        opt.step(scale=1024)
+        bc1, bc2 = oracle.bias_corrections(0.9, 0.999, step)
+        gb = bits16(g)
+        for lo in range(0, n, piece):
+            hi = min(lo + piece, n)
+            oracle.adam_cpu_fp16(po[lo:hi], ho[lo:hi], None, gb[lo:hi], mo[lo:hi], vo[lo:hi], 0.9, 0.999, 1e-8, 1e-3, 1024.0,
+                                 0.01, bc1, bc2, level, threads)
+    torch.cuda.synchronize()
+    state = opt.state[param]
+    assert state["step"] == 10
+    assert np.array_equal(f32_bits(state["_param_fp32"].numpy()), f32_bits(po))
+    assert np.array_equal(f32_bits(state["exp_avg"].numpy()), f32_bits(mo))
+    assert np.array_equal(f32_bits(state["exp_avg_sq"].numpy()), f32_bits(vo))
+    assert np.array_equal(bits16(param.detach()), ho)
+    # and the update is a real one: ten steps of lr 1e-3 with random gradients move a parameter by a few 1e-3
+    moved = (state["_param_fp32"] - master).abs()
+    assert 1e-3 < moved.mean().item() < 1e-2
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_offload_in_pieces_equals_offload_in_one_call(dtype):
     """A tensor cut into pieces (each with its own copy event) ends in the state one host call over the
