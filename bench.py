@@ -251,6 +251,27 @@ def other_workloads(torch, dev, LF, OF, iters=20):
     del x, soft
     torch.cuda.empty_cache()
 
+    # the two row helpers of the vocabulary-parallel loss, bf16, 8,192 rows x 128,256 classes
+    rows, classes = 8192, 128256
+    x = torch.empty(rows, classes, dtype=torch.bfloat16, device=dev)
+    fill_normal_(x.view(-1), 3.0, gen)
+    row_max = torch.full((rows,), 14.0, dtype=torch.float32, device=dev)
+    row_sum = torch.full((rows,), 5e4, dtype=torch.float32, device=dev)
+    out["fused_sumexp_bf16_8192x128256"] = entry(timed(lambda: LF.fused_sumexp(x, row_max)), (2 * classes + 8) * rows)
+    out["fused_softmax_inplace_bf16_8192x128256"] = entry(timed(lambda: LF.fused_softmax_inplace(x, row_max, row_sum)),
+                                                          (4 * classes + 8) * rows)
+    del x
+    torch.cuda.empty_cache()
+
+    # many small tensors through one multi-tensor launch: 300 vectors of 4,096 elements
+    small = [(torch.zeros(4096, device=dev), torch.zeros(4096, dtype=torch.bfloat16, device=dev),
+              torch.zeros(4096, dtype=torch.bfloat16, device=dev), torch.zeros(4096, device=dev), torch.zeros(4096, device=dev))
+             for _ in range(300)]
+    stats = timed(lambda: OF.adam_multi(small, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100))
+    out["adam_multi_bf16_300x4096"] = {"ms": round(stats[0], 4), "ms_median": round(stats[1], 4), "ms_min": round(stats[2], 4),
+                                       "what": "300 tensors of 4,096 elements, 32 per launch (launch-bound, not a bandwidth figure)"}
+    del small
+
     # the offload optimizer on one block: gradients device -> host, host Adam, 16-bit parameters host -> device
     import bmtrain_amd as bmt
     n = 202_383_360

@@ -21,6 +21,7 @@
 //          p' = fma(-(lr*wd), p, p - ((lr*m')/bc1) / (sqrt((v'*scale)/bc2) + eps*scale))
 // This is the reference's expression with the multiply-adds contracted the way
 // its own host compiler contracts the identical CPU loop (adam_cpu.hpp:265-276).
+#include <type_traits>
 #include "bmt_device.h"
 #include "bmt_host.h"
 #include "../../include/bmt_hip.h"
@@ -98,20 +99,6 @@ __device__ __forceinline__ void st(T *p, T v) { __builtin_nontemporal_store(v, p
 // Launch shape of the short vector kernels: one workgroup owns one tile and exits.
 constexpr int kAdamThreads = 1024;
 constexpr int kAdamUnroll = 1;
-
-// The multi-tensor kernel hands its tiles out by ticket from 8,192 tiles on: a counter in the
-// caller's 16-bit output, zeroed by a one-lane kernel in front (see adam_multi).
-__global__ void adam_ticket_reset_kernel(uint32_t *counter) { *counter = 0u; }
-
-template <bool TICKET>
-__device__ __forceinline__ int64_t adam_tile_index(uint32_t *counter) {
-    if (!TICKET) return blockIdx.x;
-    __shared__ uint32_t ticket;
-    if (threadIdx.x == 0) ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    return ticket;
-}
-constexpr int64_t kAdamTicketMinTiles = 8192;
 
 // Vector body, bf16.  `nvec` = number of 4-element groups; every pointer is aligned for its
 // vector type.  A tile is kAdamThreads * UNROLL groups; group u of a lane sits kAdamThreads groups
@@ -494,13 +481,15 @@ struct AdamBatch {
     int64_t n[kBatch];
     uint32_t first_tile[kBatch + 1];
     int32_t count;
+    // long batches (adam_stream_multi_kernel): tiles of kStreamThreads groups, vector part of each tensor only
+    uint32_t stream_first[kBatch + 1];
+    int32_t counter_tensor;     // the tensor whose 16-bit output hosts the four tile counters
 };
 
-template <bool FP16, bool TICKET>
-__global__ __launch_bounds__(kAdamThreads) void adam_multi_kernel(AdamBatch batch, AdamHyper h, uint32_t *counter) {
+template <bool FP16>
+__global__ __launch_bounds__(kAdamThreads) void adam_multi_kernel(AdamBatch batch, AdamHyper h) {
     const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
-    // the tile is the same for every lane; saying so keeps the table look-ups below on the scalar unit
-    const uint32_t tile = __builtin_amdgcn_readfirstlane((uint32_t)adam_tile_index<TICKET>(counter));
+    const uint32_t tile = blockIdx.x;
     int t = 0;
     while (t + 1 < batch.count && tile >= batch.first_tile[t + 1]) t++;
     const int64_t n = batch.n[t];
@@ -545,6 +534,124 @@ __global__ __launch_bounds__(kAdamThreads) void adam_multi_kernel(AdamBatch batc
     }
 }
 
+// ---- long batches: the resident grid over several tensors ---------------------------------------
+// The streaming scheme of adam_stream_kernel with the tile -> tensor mapping of adam_multi_kernel: tiles of
+// kStreamThreads groups are numbered through the vector parts of all tensors of the batch
+// (batch.stream_first), handed out by ticket, and each stage looks its tensor up in the kernel
+// argument (the tile is uniform, so the look-up runs on the scalar unit).  The four counters live in the
+// 16-bit output of batch.counter_tensor.  The elements that do not fill a 4-element group (up to three per
+// tensor) and the four vectors that hosted the counters are finished by adam_stream_multi_finish_kernel.
+template <bool FP16>
+__global__ __launch_bounds__(kStreamThreads) void adam_stream_multi_kernel(AdamBatch batch, AdamHyper h) {
+    typedef typename MomentVec<FP16>::type mom_t;
+    typedef StreamSet<FP16> Set;
+    const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
+    __shared__ uint32_t handed[2];
+    const int which = (int)((blockIdx.x >> 3) & (kStreamCounters - 1));
+    const int64_t ntiles = batch.stream_first[batch.count];
+    const int ct = batch.counter_tensor;
+    const int64_t ct_nvec = batch.n[ct] / 4;
+    uint32_t *counter = (uint32_t *)((u32x2 *)batch.p16[ct] + (ct_nvec - 1 - which * kStreamCounterStride));
+    if (threadIdx.x == 0) {
+        handed[0] = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        handed[1] = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    const int64_t first = (int64_t)handed[0] * kStreamCounters + which;
+    int64_t ahead = (int64_t)handed[1] * kStreamCounters + which;
+    __syncthreads();
+    if (first >= ntiles) return;
+    uint32_t drawn = 0;
+    if (threadIdx.x == 0) stream_draw(drawn, counter);
+
+    int ta = 0, tb = 0;        // tensor of the tile held in set a / set b (uniform)
+    auto issue = [&](Set &s, int &t, int64_t tile_in) {
+        const uint32_t tile = __builtin_amdgcn_readfirstlane((uint32_t)(tile_in < ntiles ? tile_in : 0));
+        t = 0;
+        while (t + 1 < batch.count && tile >= batch.stream_first[t + 1]) t++;
+        const int64_t nvec = batch.n[t] / 4;
+        s.i = (int64_t)(tile - batch.stream_first[t]) * kStreamThreads + threadIdx.x;
+        s.ok = tile_in < ntiles && s.i < nvec;
+        const int64_t j = s.ok ? s.i : 0;
+        stream_load(s.g, (const u32x2 *)batch.g16[t] + j);
+        stream_load(s.p, (const f32x4 *)batch.p32[t] + j);
+        stream_load(s.m, (const mom_t *)batch.mom[t] + j);
+        stream_load(s.v, (const f32x4 *)batch.var[t] + j);
+    };
+    auto finish = [&](Set &s, int t) {
+        if (!s.ok) return;
+        u32x2 o;
+        if constexpr (FP16) {
+            f32x4 mm = f32x4{lo_f32<Half>(s.m.x), hi_f32<Half>(s.m.x), lo_f32<Half>(s.m.y), hi_f32<Half>(s.m.y)};
+            adam_group_scaled<Half>(s.g, mm, s.v, s.p, h, omb1, omb2, lrwd, eps_s);
+            s.m = u32x2{pack2<Half>(mm.x, mm.y), pack2<Half>(mm.z, mm.w)};
+            o = u32x2{pack2<Half>(s.p.x, s.p.y), pack2<Half>(s.p.z, s.p.w)};
+        } else {
+            adam_group_unscaled<BFloat16>(s.g, s.m, s.v, s.p, h, omb1, omb2, lrwd);
+            o = u32x2{pack2<BFloat16>(s.p.x, s.p.y), pack2<BFloat16>(s.p.z, s.p.w)};
+        }
+        stream_store((f32x4 *)batch.p32[t] + s.i, s.p);
+        stream_store((mom_t *)batch.mom[t] + s.i, s.m);
+        stream_store((f32x4 *)batch.var[t] + s.i, s.v);
+        if (!(t == ct && holds_stream_counter(s.i, ct_nvec))) stream_store((u32x2 *)batch.p16[t] + s.i, o);
+    };
+    auto stage = [&](Set &cur, int tcur, Set &next, int &tnext, int slot) -> int64_t {
+        const int64_t tile = ahead;
+        issue(next, tnext, tile);
+        asm volatile("s_waitcnt vmcnt(4)" : "+v"(cur.g), "+v"(cur.p), "+v"(cur.m), "+v"(cur.v), "+v"(drawn));
+        if (threadIdx.x == 0) handed[slot] = drawn;
+        __syncthreads();
+        ahead = (int64_t)handed[slot] * kStreamCounters + which;
+        if (threadIdx.x == 0) stream_draw(drawn, counter);
+        finish(cur, tcur);
+        return tile;
+    };
+    Set a, b;
+    issue(a, ta, first);
+    while (true) {
+        if (stage(a, ta, b, tb, 0) >= ntiles) break;
+        if (stage(b, tb, a, ta, 1) >= ntiles) break;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+}
+
+// One workgroup: lanes 0..3 write the four 16-bit vectors that hosted the counters (from the fp32 parameters
+// just written); lane 4 * t + k steps leftover element k of tensor t.
+template <bool FP16>
+__global__ __launch_bounds__(4 * kBatch + 64) void adam_stream_multi_finish_kernel(AdamBatch batch, AdamHyper h) {
+    typedef typename std::conditional<FP16, Half, BFloat16>::type T;
+    const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
+    const int lane = threadIdx.x;
+    if (lane < kStreamCounters) {
+        const int ct = batch.counter_tensor;
+        const int64_t i = batch.n[ct] / 4 - 1 - lane * kStreamCounterStride;
+        const f32x4 p = ((const f32x4 *)batch.p32[ct])[i];
+        ((u32x2 *)batch.p16[ct])[i] = u32x2{pack2<T>(p.x, p.y), pack2<T>(p.z, p.w)};
+    }
+    const int t = (lane - 64) / 4, k = (lane - 64) % 4;
+    if (lane >= 64 && t < batch.count) {
+        const int64_t n = batch.n[t], e = (n / 4) * 4 + k;
+        if (e < n) {
+            float *p32 = batch.p32[t], *var = batch.var[t];
+            uint16_t *p16 = batch.p16[t];
+            const uint16_t *g16 = batch.g16[t];
+            float p = p32[e], v = var[e];
+            if (FP16) {
+                uint16_t *mom = (uint16_t *)batch.mom[t];
+                float m = Half::to_f32(mom[e]);
+                adam_elem_scaled(clip16<Half>(Half::to_f32(g16[e]), h.gcoef), m, v, p, h, omb1, omb2, lrwd, eps_s);
+                mom[e] = Half::from_f32(m); p16[e] = Half::from_f32(p);
+            } else {
+                float *mom = (float *)batch.mom[t];
+                float m = mom[e];
+                adam_elem_unscaled(clip16<BFloat16>(BFloat16::to_f32(g16[e]), h.gcoef), m, v, p, h, omb1, omb2, lrwd);
+                mom[e] = m; p16[e] = BFloat16::from_f32(p);
+            }
+            p32[e] = p; var[e] = v;
+        }
+    }
+}
+
 // Tiles of one tensor: its 4-element groups plus one lane per leftover element.
 static int64_t multi_tiles(int64_t n) { return (n / 4 + (n % 4) + kAdamThreads - 1) / kAdamThreads; }
 
@@ -556,18 +663,24 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
     auto flush = [&]() -> hipError_t {
         if (batch.count == 0) return hipSuccess;
         const uint32_t tiles = batch.first_tile[batch.count];
-        // Long launches hand tiles out by ticket, like the single-tensor kernels.  The counter sits in the
-        // first 16-bit output vector of the last tile of the last tensor, which the workgroup with the last
-        // ticket overwrites; a last tile that holds leftover elements only has no such vector.
-        const int last = batch.count - 1;
-        const int64_t last_first_vec = (int64_t)(tiles - 1 - batch.first_tile[last]) * kAdamThreads;
-        if ((int64_t)tiles >= kAdamTicketMinTiles && last_first_vec < batch.n[last] / 4) {
-            uint32_t *counter = (uint32_t *)((u32x2 *)batch.p16[last] + last_first_vec);
-            hipLaunchKernelGGL(adam_ticket_reset_kernel, dim3(1), dim3(1), 0, s, counter);
-            hipLaunchKernelGGL((adam_multi_kernel<FP16, true>), dim3(tiles), dim3(kAdamThreads), 0, s, batch, h, counter);
+        // Batches of 2^22 groups or more run as the resident grid; the tensor with the most groups (at least
+        // 2^22 / 32 of them, so the four counter places exist) lends its 16-bit output to the counters.
+        int64_t groups = 0, most = -1;
+        batch.stream_first[0] = 0;
+        batch.counter_tensor = 0;
+        for (int c = 0; c < batch.count; c++) {
+            const int64_t nvec = batch.n[c] / 4;
+            groups += nvec;
+            if (nvec > most) { most = nvec; batch.counter_tensor = c; }
+            batch.stream_first[c + 1] = batch.stream_first[c] + (uint32_t)((nvec + kStreamThreads - 1) / kStreamThreads);
+        }
+        if (groups >= kStreamMinVec) {
+            hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, (u32x2 *)batch.p16[batch.counter_tensor], most);
+            hipLaunchKernelGGL((adam_stream_multi_kernel<FP16>), dim3((unsigned)device_cu_count()), dim3(kStreamThreads), 0, s,
+                               batch, h);
+            hipLaunchKernelGGL((adam_stream_multi_finish_kernel<FP16>), dim3(1), dim3(4 * kBatch + 64), 0, s, batch, h);
         } else {
-            hipLaunchKernelGGL((adam_multi_kernel<FP16, false>), dim3(tiles), dim3(kAdamThreads), 0, s, batch, h,
-                               (uint32_t *)nullptr);
+            hipLaunchKernelGGL((adam_multi_kernel<FP16>), dim3(tiles), dim3(kAdamThreads), 0, s, batch, h);
         }
         batch.count = 0;
         batch.first_tile[0] = 0;
@@ -584,7 +697,7 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
         const bool aligned = (((uintptr_t)t.param_fp32 | (uintptr_t)t.v | (FP16 ? 0 : (uintptr_t)t.m)) & 15u) == 0 &&
                              (((uintptr_t)t.param_16 | (uintptr_t)t.grad_16 | (FP16 ? (uintptr_t)t.m : 0)) & 7u) == 0;
         const int64_t tiles = multi_tiles(t.n);
-        if (!aligned || tiles > 0x3FFFFFFF) {
+        if (!aligned || tiles > 0x0FFFFFFF) {
             // tensors the batch kernel does not take (unaligned views, gigantic buffers) go alone
             hipError_t e = FP16 ? launch_fp16(t.n, (float *)t.param_fp32, (uint16_t *)t.param_16, (const uint16_t *)t.grad_16,
                                               (uint16_t *)t.m, (float *)t.v, h, s)
@@ -593,7 +706,7 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
             if (e != hipSuccess) return fail((int)e, who, e);
             continue;
         }
-        if (batch.count == kBatch || (int64_t)batch.first_tile[batch.count] + tiles > 0x7FFFFFFF) {
+        if (batch.count == kBatch || (int64_t)batch.first_tile[batch.count] + tiles > 0x0FFFFFFF) {
             hipError_t e = flush();
             if (e != hipSuccess) return fail((int)e, who, e);
         }

@@ -40,13 +40,12 @@ class AdamOptimizer(torch.optim.Optimizer):
         validate_hyper(lr, betas, eps, weight_decay)
         super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
         self._hold_steps = hold_steps
-        # Tensors below `batch_below` elements share launches (same arithmetic per element as one launch per
-        # tensor, which remains available by setting batch_launches to False).  Larger tensors keep a launch
-        # of their own unless the tensors that could share launches hold `batch_all_from` elements or more.
+        # Tensors share launches, up to 32 per launch (same arithmetic per element as one launch per tensor,
+        # which remains available by setting batch_launches to False); a batch of 2^24 elements or more runs as
+        # one resident grid over all its tensors.  Tensors of `alone_from` elements or more are long launches
+        # by themselves.
         self.batch_launches = True
-        self.batch_below = 1 << 20
-        self.batch_all_from = 1 << 26
-        self.ticket_alone = 1 << 28
+        self.alone_from = 1 << 28
         # Parameters, gradients and state that are adjacent in memory are stepped as one flat tensor.
         self.merge_adjacent = True
 
@@ -134,9 +133,7 @@ class AdamOptimizer(torch.optim.Optimizer):
                     lr = 0.0 if state["step"] < self._hold_steps else group["lr"]
                     half.append((state["_param_fp32"], p, grad, state["exp_avg"], state["exp_avg_sq"], state["step"], lr))
 
-            # 16-bit parameters that can share launches: (dtype, step, lr) -> tensors.  Small tensors always
-            # do; when a class holds enough elements for tiles to be handed out by ticket (where one long
-            # launch beats many medium ones), the large tensors join it too.
+            # 16-bit parameters that can share launches: (dtype, step, lr) -> tensors.
             batches, singles = {}, []
             coef16 = {}
             if grad_coef is not None:      # the factor as the in-place multiplication would see it, per dtype
@@ -153,11 +150,8 @@ class AdamOptimizer(torch.optim.Optimizer):
                 else:
                     singles.append(item)
             for key in list(batches) if not coef16 else []:     # with a clipping factor everything goes batched
-                # tensors of `ticket_alone` elements or more are long launches by themselves
-                shared = [w for w in batches[key] if w[1].numel() < self.ticket_alone]
-                limit = self.ticket_alone if sum(w[1].numel() for w in shared) >= self.batch_all_from else self.batch_below
-                singles.extend(w for w in batches[key] if w[1].numel() >= limit)
-                batches[key] = [w for w in batches[key] if w[1].numel() < limit]
+                singles.extend(w for w in batches[key] if w[1].numel() >= self.alone_from)
+                batches[key] = [w for w in batches[key] if w[1].numel() < self.alone_from]
             for p32, p, grad, m, v, step, lr in singles:
                 if coef16:                 # not contiguous: clip a copy of the gradient eagerly
                     grad = grad * torch.as_tensor(grad_coef, dtype=torch.float32, device=grad.device)

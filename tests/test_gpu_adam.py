@@ -354,14 +354,17 @@ def test_multi_tensor_launch_equals_per_tensor_launches(flavour):
 
 
 @pytest.mark.parametrize("flavour", ["bf16", "fp16"])
-def test_long_multi_tensor_launch_hands_tiles_out_by_ticket(flavour):
-    """Batches of 8,192 tiles or more draw tiles from a counter kept in the last tensor's 16-bit output.
-    40 tensors (two launches), bit for bit against one launch per tensor; a second table ends in a tensor
-    whose last tile holds leftover elements only (no room for the counter: workgroup-id order)."""
+def test_long_multi_tensor_launch_runs_as_one_resident_grid(flavour):
+    """Batches of 2^24 elements or more run as one resident grid over all their tensors: tiles of 256 groups numbered
+    through the tensors, drawn by ticket from four counters kept in the 16-bit output of the largest tensor; leftover
+    elements and the counters' places are finished by a small kernel.  40 tensors (two launches, the second a short
+    one), 33 equal tensors, and a mix of sizes from 3 to 2^24 + 5 elements with every leftover count — bit for bit
+    against one launch per tensor."""
     dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
     mdt = torch.float16 if flavour == "fp16" else torch.float32
     fn = F.adam_fp16 if flavour == "fp16" else F.adam_bf16
-    for sizes in ([1_200_001 + 4 * k for k in range(39)] + [2_000_003], [1_200_000] * 32 + [4096 * 300 + 3]):
+    for sizes in ([1_200_001 + 4 * k for k in range(39)] + [2_000_003], [1_200_000] * 32 + [4096 * 300 + 3],
+                  [(1 << 24) + 5, 77, 4096, (1 << 22) + 2, 3, 1_000_001, 255, 1024, 1023, 6, (1 << 23) + 3]):
         gen = torch.Generator(device="cuda").manual_seed(len(sizes))
         single, multi = [], []
         for n in sizes:
