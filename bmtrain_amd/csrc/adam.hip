@@ -67,14 +67,22 @@ __device__ __forceinline__ void adam_elem_scaled(float g, float &m, float &v, fl
     m = mm; v = vv; p = np;
 }
 
+// The same for the four packed gradients of a group, with the hardware's packed round-to-nearest-even converts.
+template <typename T>
+__device__ __forceinline__ u32x2 clip_group(u32x2 g, float coef) {
+    if (coef == 1.0f) return g;
+    return u32x2{pack2<T>(lo_f32<T>(g.x) * coef, hi_f32<T>(g.x) * coef), pack2<T>(lo_f32<T>(g.y) * coef, hi_f32<T>(g.y) * coef)};
+}
+
 // Four elements at once: gradients arrive as two packed dwords.
 template <typename T>
 __device__ __forceinline__ void adam_group_unscaled(u32x2 g, f32x4 &m, f32x4 &v, f32x4 &p, const AdamHyper &h, float omb1,
                                                     float omb2, float lrwd) {
+    g = clip_group<T>(g, h.gcoef);
     float gm[4] = {lo_f32<T>(g.x), hi_f32<T>(g.x), lo_f32<T>(g.y), hi_f32<T>(g.y)};
     float ma[4] = {m.x, m.y, m.z, m.w}, va[4] = {v.x, v.y, v.z, v.w}, pa[4] = {p.x, p.y, p.z, p.w};
 #pragma unroll
-    for (int k = 0; k < 4; k++) adam_elem_unscaled(clip16<T>(gm[k], h.gcoef), ma[k], va[k], pa[k], h, omb1, omb2, lrwd);
+    for (int k = 0; k < 4; k++) adam_elem_unscaled(gm[k], ma[k], va[k], pa[k], h, omb1, omb2, lrwd);
     m = f32x4{ma[0], ma[1], ma[2], ma[3]};
     v = f32x4{va[0], va[1], va[2], va[3]};
     p = f32x4{pa[0], pa[1], pa[2], pa[3]};
@@ -82,10 +90,11 @@ __device__ __forceinline__ void adam_group_unscaled(u32x2 g, f32x4 &m, f32x4 &v,
 template <typename T>
 __device__ __forceinline__ void adam_group_scaled(u32x2 g, f32x4 &m, f32x4 &v, f32x4 &p, const AdamHyper &h, float omb1,
                                                   float omb2, float lrwd, float eps_s) {
+    g = clip_group<T>(g, h.gcoef);
     float gm[4] = {lo_f32<T>(g.x), hi_f32<T>(g.x), lo_f32<T>(g.y), hi_f32<T>(g.y)};
     float ma[4] = {m.x, m.y, m.z, m.w}, va[4] = {v.x, v.y, v.z, v.w}, pa[4] = {p.x, p.y, p.z, p.w};
 #pragma unroll
-    for (int k = 0; k < 4; k++) adam_elem_scaled(clip16<T>(gm[k], h.gcoef), ma[k], va[k], pa[k], h, omb1, omb2, lrwd, eps_s);
+    for (int k = 0; k < 4; k++) adam_elem_scaled(gm[k], ma[k], va[k], pa[k], h, omb1, omb2, lrwd, eps_s);
     m = f32x4{ma[0], ma[1], ma[2], ma[3]};
     v = f32x4{va[0], va[1], va[2], va[3]};
     p = f32x4{pa[0], pa[1], pa[2], pa[3]};
@@ -564,21 +573,36 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_multi_kernel(AdamB
     uint32_t drawn = 0;
     if (threadIdx.x == 0) stream_draw(drawn, counter);
 
-    int ta = 0, tb = 0;        // tensor of the tile held in set a / set b (uniform)
-    auto issue = [&](Set &s, int &t, int64_t tile_in) {
-        const uint32_t tile = __builtin_amdgcn_readfirstlane((uint32_t)(tile_in < ntiles ? tile_in : 0));
-        t = 0;
-        while (t + 1 < batch.count && tile >= batch.stream_first[t + 1]) t++;
-        const int64_t nvec = batch.n[t] / 4;
-        s.i = (int64_t)(tile - batch.stream_first[t]) * kStreamThreads + threadIdx.x;
-        s.ok = tile_in < ntiles && s.i < nvec;
-        const int64_t j = s.ok ? s.i : 0;
-        stream_load(s.g, (const u32x2 *)batch.g16[t] + j);
-        stream_load(s.p, (const f32x4 *)batch.p32[t] + j);
-        stream_load(s.m, (const mom_t *)batch.mom[t] + j);
-        stream_load(s.v, (const f32x4 *)batch.var[t] + j);
+    // The tiles a workgroup draws only ever go up, so the tensor of a tile is found by walking on from the
+    // tensor of the tile before, and its pointers are read from the kernel argument only when it changes;
+    // each register set remembers the pointers its tile was loaded through.
+    struct Where { float *p32; uint16_t *p16; const uint16_t *g16; void *mom; float *var; int64_t nvec; bool hosts_counters; };
+    int t = 0;
+    uint32_t t_first = 0, t_end = batch.stream_first[1];       // tensor t owns the tiles [t_first, t_end)
+    auto where_of = [&](int k) {
+        return Where{batch.p32[k], batch.p16[k], batch.g16[k], batch.mom[k], batch.var[k], batch.n[k] / 4, k == ct};
     };
-    auto finish = [&](Set &s, int t) {
+    Where cur_where = where_of(0), wa = cur_where, wb = cur_where;
+    auto issue = [&](Set &s, Where &w, int64_t tile_in) {
+        const bool real = tile_in < ntiles;
+        if (real) {
+            const uint32_t tile = __builtin_amdgcn_readfirstlane((uint32_t)tile_in);
+            bool moved = false;
+            while (tile >= t_end) { t++; t_first = t_end; t_end = batch.stream_first[t + 1]; moved = true; }
+            if (moved) cur_where = where_of(t);
+            s.i = (int64_t)(tile - t_first) * kStreamThreads + threadIdx.x;
+        } else {
+            s.i = 0;
+        }
+        w = cur_where;
+        s.ok = real && s.i < w.nvec;
+        const int64_t j = s.ok ? s.i : 0;          // lanes without a group load group 0 of some tensor and drop it
+        stream_load(s.g, (const u32x2 *)w.g16 + j);
+        stream_load(s.p, (const f32x4 *)w.p32 + j);
+        stream_load(s.m, (const mom_t *)w.mom + j);
+        stream_load(s.v, (const f32x4 *)w.var + j);
+    };
+    auto finish = [&](Set &s, const Where &w) {
         if (!s.ok) return;
         u32x2 o;
         if constexpr (FP16) {
@@ -590,27 +614,27 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_multi_kernel(AdamB
             adam_group_unscaled<BFloat16>(s.g, s.m, s.v, s.p, h, omb1, omb2, lrwd);
             o = u32x2{pack2<BFloat16>(s.p.x, s.p.y), pack2<BFloat16>(s.p.z, s.p.w)};
         }
-        stream_store((f32x4 *)batch.p32[t] + s.i, s.p);
-        stream_store((mom_t *)batch.mom[t] + s.i, s.m);
-        stream_store((f32x4 *)batch.var[t] + s.i, s.v);
-        if (!(t == ct && holds_stream_counter(s.i, ct_nvec))) stream_store((u32x2 *)batch.p16[t] + s.i, o);
+        stream_store((f32x4 *)w.p32 + s.i, s.p);
+        stream_store((mom_t *)w.mom + s.i, s.m);
+        stream_store((f32x4 *)w.var + s.i, s.v);
+        if (!(w.hosts_counters && holds_stream_counter(s.i, ct_nvec))) stream_store((u32x2 *)w.p16 + s.i, o);
     };
-    auto stage = [&](Set &cur, int tcur, Set &next, int &tnext, int slot) -> int64_t {
+    auto stage = [&](Set &cur, const Where &wcur, Set &next, Where &wnext, int slot) -> int64_t {
         const int64_t tile = ahead;
-        issue(next, tnext, tile);
+        issue(next, wnext, tile);
         asm volatile("s_waitcnt vmcnt(4)" : "+v"(cur.g), "+v"(cur.p), "+v"(cur.m), "+v"(cur.v), "+v"(drawn));
         if (threadIdx.x == 0) handed[slot] = drawn;
         __syncthreads();
         ahead = (int64_t)handed[slot] * kStreamCounters + which;
         if (threadIdx.x == 0) stream_draw(drawn, counter);
-        finish(cur, tcur);
+        finish(cur, wcur);
         return tile;
     };
     Set a, b;
-    issue(a, ta, first);
+    issue(a, wa, first);
     while (true) {
-        if (stage(a, ta, b, tb, 0) >= ntiles) break;
-        if (stage(b, tb, a, ta, 1) >= ntiles) break;
+        if (stage(a, wa, b, wb, 0) >= ntiles) break;
+        if (stage(b, wb, a, wa, 1) >= ntiles) break;
     }
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
 }

@@ -61,16 +61,18 @@ class State:
     """in_flight: VGPR -> least number of vector-memory operations issued behind its load.
     exec_nz: the exec mask is known to be non-zero.  nz: SGPR pairs known to hold a non-zero mask."""
 
-    def __init__(self, in_flight=None, exec_nz=True, nz=frozenset()):
+    def __init__(self, in_flight=None, exec_nz=True, nz=frozenset(), ones=frozenset(), vcc_nz=False):
         self.in_flight = dict(in_flight or {})
         self.exec_nz = exec_nz
         self.nz = frozenset(nz)
+        self.ones = frozenset(ones)      # SGPR pairs known to hold -1
+        self.vcc_nz = vcc_nz             # vcc is known to be non-zero
 
     def key(self):
-        return (tuple(sorted(self.in_flight.items())), self.exec_nz, self.nz)
+        return (tuple(sorted(self.in_flight.items())), self.exec_nz, self.nz, self.ones, self.vcc_nz)
 
     def copy(self):
-        return State(self.in_flight, self.exec_nz, self.nz)
+        return State(self.in_flight, self.exec_nz, self.nz, self.ones, self.vcc_nz)
 
 
 def merge(a, b):
@@ -79,12 +81,13 @@ def merge(a, b):
     out = dict(a.in_flight)
     for r, k in b.in_flight.items():
         out[r] = min(out[r], k) if r in out else k
-    return State(out, a.exec_nz and b.exec_nz, a.nz & b.nz)
+    return State(out, a.exec_nz and b.exec_nz, a.nz & b.nz, a.ones & b.ones, a.vcc_nz and b.vcc_nz)
 
 
 def successors(insts, labels, i, state):
     """Where control can go after instruction i.  A branch on `exec == 0` is not followed when the mask
-    is known to be non-zero (the compiler emits such branches around uniform loop exits)."""
+    is known to be non-zero, nor one on vcc when vcc is known to be `exec & -1` with exec non-zero (the compiler
+    emits both around uniform loop exits)."""
     text = insts[i]
     op = text.split()[0]
     if op == "s_endpgm":
@@ -95,6 +98,10 @@ def successors(insts, labels, i, state):
         return [i + 1] if state.exec_nz else [labels[text.split()[1]], i + 1]
     if op == "s_cbranch_execnz":
         return [labels[text.split()[1]]] if state.exec_nz else [labels[text.split()[1]], i + 1]
+    if op == "s_cbranch_vccnz" and state.vcc_nz:
+        return [labels[text.split()[1]]]
+    if op == "s_cbranch_vccz" and state.vcc_nz:
+        return [i + 1]
     if op.startswith("s_cbranch"):
         return [labels[text.split()[1]], i + 1]
     return [i + 1]
@@ -107,11 +114,21 @@ def is_vmem(op):
 def scalar_effects(text, st):
     """Tracks whether exec is known non-zero through the save / restore idiom of divergent branches."""
     op = text.split()[0]
-    if not op.startswith("s_"):
-        return
     parts = [p.strip() for p in text[len(op):].split(",")]
     dest = parts[0] if parts else ""
     pairs = lambda t: {int(m.group(1)) for m in SREG_PAIR.finditer(t)}
+    # vcc: known non-zero only right after `s_and_b64 vcc, exec, <pair holding -1>` with exec non-zero; anything
+    # else that may write it (every mention outside pure readers, every v_cmp) makes it unknown again
+    if op == "s_and_b64" and dest == "vcc" and parts[1] == "exec" and pairs(parts[2]) & st.ones and st.exec_nz:
+        st.vcc_nz = True
+    elif op.startswith("v_cmp") or ("vcc" in text and not op.startswith(("s_cbranch", "v_cndmask", "v_div_fmas"))):
+        st.vcc_nz = False
+    if not op.startswith("s_"):
+        return
+    if op == "s_mov_b64" and dest != "exec" and parts[1] == "-1":
+        st.ones = st.ones | pairs(dest)
+    elif pairs(dest) & st.ones:
+        st.ones = st.ones - pairs(dest)
     if op == "s_and_saveexec_b64" or op == "s_or_saveexec_b64":
         saved = pairs(dest)
         st.nz = (st.nz - saved) | (saved if st.exec_nz else set())
@@ -134,6 +151,7 @@ def scalar_effects(text, st):
     if m:
         n = int(m.group(1))
         st.nz = frozenset(x for x in st.nz if x != n and x + 1 != n)
+        st.ones = frozenset(x for x in st.ones if x != n and x + 1 != n)
 
 
 def transfer(text, st, where, problems):
@@ -192,26 +210,40 @@ def store_data_hazards(insts, name):
 
 
 def check(lines, start, name):
+    """Forward data-flow.  States that differ in what is known about scalar registers (exec, vcc, pairs holding
+    -1 or a non-zero mask) are kept apart at joins, so that a branch decided by such a fact on one incoming path
+    only is followed correctly; states that agree in those facts are merged."""
     insts, labels = parse_kernel(lines, start)
-    state_in = [None] * (len(insts) + 1)
-    state_in[0] = State()
-    work = [0]
+    facts = lambda st: (st.exec_nz, st.nz, st.ones, st.vcc_nz)
+    state_in = [dict() for _ in range(len(insts) + 1)]
+    state_in[0][facts(State())] = State()
+    work = [(0, facts(State()))]
+    steps = 0
     while work:
-        i = work.pop()
-        if i >= len(insts):
+        i, f = work.pop()
+        steps += 1
+        if i >= len(insts) or steps > 2_000_000:
             continue
-        out = transfer(insts[i], state_in[i].copy(), "", [])
+        out = transfer(insts[i], state_in[i][f].copy(), "", [])
         for j in successors(insts, labels, i, out):
-            merged = merge(state_in[j], out)
-            if state_in[j] is None or merged.key() != state_in[j].key():
-                state_in[j] = merged
-                work.append(j)
+            fj = facts(out)
+            merged = merge(state_in[j].get(fj), out)
+            if fj not in state_in[j] or merged.key() != state_in[j][fj].key():
+                state_in[j][fj] = merged
+                work.append((j, fj))
     problems = store_data_hazards(insts, name)
+    if steps > 2_000_000:
+        problems.append(f"{name}: analysis did not converge")
+    seen = set()
     loads = waits = 0
     for i, text in enumerate(insts):
-        if state_in[i] is None:
-            continue
-        transfer(text, state_in[i].copy(), f"{name} instruction {i}", problems)
+        for st in state_in[i].values():
+            found = []
+            transfer(text, st.copy(), f"{name} instruction {i}", found)
+            for msg in found:
+                if msg not in seen:
+                    seen.add(msg)
+                    problems.append(msg)
         loads += text.startswith("global_load")
         waits += text.startswith("s_waitcnt") and "vmcnt" in text
     return problems, len(insts), loads, waits
