@@ -214,8 +214,24 @@ __device__ __forceinline__ bool holds_stream_counter(int64_t i, int64_t nvec) {
     const int64_t d = nvec - 1 - i;
     return (d & (kStreamCounterStride - 1)) == 0 && d < kStreamCounters * kStreamCounterStride;
 }
-__global__ void adam_stream_reset_kernel(u32x2 *p16, int64_t nvec) {
-    if (threadIdx.x < kStreamCounters) p16[nvec - 1 - threadIdx.x * kStreamCounterStride] = u32x2{0u, 0u};
+// Every workgroup starts on two tiles it can name itself (see stream_first_tickets), so the counters
+// start at twice the number of workgroups that share a counter.
+__global__ void adam_stream_reset_kernel(u32x2 *p16, int64_t nvec, uint32_t first_ticket) {
+    if (threadIdx.x < kStreamCounters) p16[nvec - 1 - threadIdx.x * kStreamCounterStride] = u32x2{first_ticket, 0u};
+}
+// The grid of the resident kernels: one workgroup per compute unit, rounded down to a multiple of 32
+// (8 XCDs x 4 counters), at least 32.
+static unsigned stream_grid() {
+    const int cus = device_cu_count();
+    return (unsigned)(cus >= 32 ? cus / 32 * 32 : 32);
+}
+// Workgroup b draws from counter (b / 8) % 4.  Its first two tickets need no atomic: it is workgroup number q
+// among the gridDim / 4 that share the counter, and takes tickets q and q + gridDim / 4.
+__device__ __forceinline__ void stream_first_tickets(int &which, uint32_t &t0, uint32_t &t1) {
+    which = (int)((blockIdx.x >> 3) & (kStreamCounters - 1));
+    const uint32_t q = ((blockIdx.x >> 5) << 3) | (blockIdx.x & 7u);
+    t0 = q;
+    t1 = q + (gridDim.x >> 2);
 }
 template <typename T>
 __global__ void adam_stream_finish_kernel(const f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, int64_t nvec) {
@@ -261,16 +277,12 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_kernel(
     typedef StreamSet<FP16> Set;
     const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
     __shared__ uint32_t handed[2];
-    const int which = (int)((blockIdx.x >> 3) & (kStreamCounters - 1));
+    int which;
+    uint32_t t0, t1;
+    stream_first_tickets(which, t0, t1);
     uint32_t *counter = (uint32_t *)(p16 + (nvec - 1 - which * kStreamCounterStride));
-    if (threadIdx.x == 0) {
-        handed[0] = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        handed[1] = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    const int64_t first = (int64_t)handed[0] * kStreamCounters + which;
-    int64_t ahead = (int64_t)handed[1] * kStreamCounters + which;     // the tile after the one in flight
-    __syncthreads();
+    const int64_t first = (int64_t)t0 * kStreamCounters + which;
+    int64_t ahead = (int64_t)t1 * kStreamCounters + which;            // the tile after the one in flight
     if (first >= ntiles) return;
     uint32_t drawn = 0;                                               // lane 0: ticket on its way
     if (threadIdx.x == 0) stream_draw(drawn, counter);
@@ -424,8 +436,8 @@ static hipError_t launch_bf16(int64_t n, float *p32, uint16_t *p16, const uint16
             u32x2 *out16 = (u32x2 *)(p16 + head);
             if (nvec >= kStreamMinVec) {
                 const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
-                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec);
-                hipLaunchKernelGGL((adam_stream_kernel<false>), dim3((unsigned)device_cu_count()), dim3(kStreamThreads), 0, s, nvec,
+                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec, stream_grid() / 2);
+                hipLaunchKernelGGL((adam_stream_kernel<false>), dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
                                    ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (f32x4 *)(m + head),
                                    (f32x4 *)(v + head), h);
                 hipLaunchKernelGGL((adam_stream_finish_kernel<BFloat16>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
@@ -454,8 +466,8 @@ static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16
             u32x2 *out16 = (u32x2 *)(p16 + head);
             if (nvec >= kStreamMinVec) {
                 const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
-                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec);
-                hipLaunchKernelGGL((adam_stream_kernel<true>), dim3((unsigned)device_cu_count()), dim3(kStreamThreads), 0, s, nvec,
+                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec, stream_grid() / 2);
+                hipLaunchKernelGGL((adam_stream_kernel<true>), dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
                                    ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
                                    (f32x4 *)(v + head), h);
                 hipLaunchKernelGGL((adam_stream_finish_kernel<Half>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
@@ -556,19 +568,15 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_multi_kernel(AdamB
     typedef StreamSet<FP16> Set;
     const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
     __shared__ uint32_t handed[2];
-    const int which = (int)((blockIdx.x >> 3) & (kStreamCounters - 1));
+    int which;
+    uint32_t t0, t1;
+    stream_first_tickets(which, t0, t1);
     const int64_t ntiles = batch.stream_first[batch.count];
     const int ct = batch.counter_tensor;
     const int64_t ct_nvec = batch.n[ct] / 4;
     uint32_t *counter = (uint32_t *)((u32x2 *)batch.p16[ct] + (ct_nvec - 1 - which * kStreamCounterStride));
-    if (threadIdx.x == 0) {
-        handed[0] = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        handed[1] = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    const int64_t first = (int64_t)handed[0] * kStreamCounters + which;
-    int64_t ahead = (int64_t)handed[1] * kStreamCounters + which;
-    __syncthreads();
+    const int64_t first = (int64_t)t0 * kStreamCounters + which;
+    int64_t ahead = (int64_t)t1 * kStreamCounters + which;
     if (first >= ntiles) return;
     uint32_t drawn = 0;
     if (threadIdx.x == 0) stream_draw(drawn, counter);
@@ -699,8 +707,9 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
             batch.stream_first[c + 1] = batch.stream_first[c] + (uint32_t)((nvec + kStreamThreads - 1) / kStreamThreads);
         }
         if (groups >= kStreamMinVec) {
-            hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, (u32x2 *)batch.p16[batch.counter_tensor], most);
-            hipLaunchKernelGGL((adam_stream_multi_kernel<FP16>), dim3((unsigned)device_cu_count()), dim3(kStreamThreads), 0, s,
+            hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, (u32x2 *)batch.p16[batch.counter_tensor], most,
+                               stream_grid() / 2);
+            hipLaunchKernelGGL((adam_stream_multi_kernel<FP16>), dim3(stream_grid()), dim3(kStreamThreads), 0, s,
                                batch, h);
             hipLaunchKernelGGL((adam_stream_multi_finish_kernel<FP16>), dim3(1), dim3(4 * kBatch + 64), 0, s, batch, h);
         } else {
