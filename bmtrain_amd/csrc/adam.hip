@@ -253,23 +253,6 @@ struct StreamSet {
     bool ok;        // the group exists
 };
 
-__device__ __forceinline__ void stream_load(f32x4 &dst, const f32x4 *src) {
-    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(src) : "memory");
-}
-__device__ __forceinline__ void stream_load(u32x2 &dst, const u32x2 *src) {
-    asm volatile("global_load_dwordx2 %0, %1, off nt" : "=v"(dst) : "v"(src) : "memory");
-}
-__device__ __forceinline__ void stream_store(f32x4 *dst, const f32x4 &v) {
-    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(dst), "v"(v) : "memory");
-}
-__device__ __forceinline__ void stream_store(u32x2 *dst, const u32x2 &v) {
-    asm volatile("global_store_dwordx2 %0, %1, off nt" : : "v"(dst), "v"(v) : "memory");
-}
-__device__ __forceinline__ void stream_draw(uint32_t &ticket, uint32_t *counter) {
-    const uint32_t one = 1u;
-    asm volatile("global_atomic_add %0, %1, %2, off sc0" : "=v"(ticket) : "v"(counter), "v"(one) : "memory");
-}
-
 template <bool FP16>
 __global__ __launch_bounds__(kStreamThreads) void adam_stream_kernel(
     int64_t nvec, int64_t ntiles, f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, const u32x2 *__restrict__ g16,

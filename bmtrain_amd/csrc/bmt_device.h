@@ -98,4 +98,33 @@ __device__ __forceinline__ float block_allreduce(float v, float *slots) {
     return r;
 }
 
+// ---- vector memory instructions of the resident streaming kernels ---------------------------
+// Those kernels keep one tile of loads in flight while they compute and store the tile before, which
+// the compiler's wait-count insertion cannot express; their loads, stores and ticket atomics are asm
+// statements and they place `s_waitcnt vmcnt(N)` themselves (see adam.hip).  A 16-byte store is
+// followed by `s_nop 1`: it reads its data registers for two more cycles, and the compiler pads that
+// hazard only for stores it emits itself.
+__device__ __forceinline__ void stream_load(f32x4 &dst, const f32x4 *src) {
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(src) : "memory");
+}
+__device__ __forceinline__ void stream_load(u32x2 &dst, const u32x2 *src) {
+    asm volatile("global_load_dwordx2 %0, %1, off nt" : "=v"(dst) : "v"(src) : "memory");
+}
+__device__ __forceinline__ void stream_store(f32x4 *dst, const f32x4 &v) {
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(dst), "v"(v) : "memory");
+}
+__device__ __forceinline__ void stream_store(u32x2 *dst, const u32x2 &v) {
+    asm volatile("global_store_dwordx2 %0, %1, off nt" : : "v"(dst), "v"(v) : "memory");
+}
+__device__ __forceinline__ void stream_load(u32x4 &dst, const u32x4 *src) {
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(src) : "memory");
+}
+__device__ __forceinline__ void stream_store(u32x4 *dst, const u32x4 &v) {
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(dst), "v"(v) : "memory");
+}
+__device__ __forceinline__ void stream_draw(uint32_t &ticket, uint32_t *counter) {
+    const uint32_t one = 1u;
+    asm volatile("global_atomic_add %0, %1, %2, off sc0" : "=v"(ticket) : "v"(counter), "v"(one) : "memory");
+}
+
 }  // namespace bmt

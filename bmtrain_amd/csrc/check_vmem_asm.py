@@ -43,14 +43,14 @@ def parse_kernel(lines, start):
     insts, labels = [], {}
     for raw in lines[start + 1:]:
         text = raw.split(";")[0].strip()
+        if raw.startswith(".Lfunc_end"):
+            break
         if raw.startswith(".LBB") or re.match(r"^\.L\w+:", raw):
             labels[raw.split(":")[0].strip()] = len(insts)
             continue
         if not text or text.startswith(".") or text.startswith(";"):
             continue
         insts.append(text)
-        if text.startswith("s_endpgm"):
-            break
     return insts, labels
 
 

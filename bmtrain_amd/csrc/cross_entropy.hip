@@ -23,6 +23,7 @@
 // Backward (reference kernels :46-60, :104-121), element-wise and in place on the
 // stored softmax: x[r, i] = to16((x[r, i] - (i == target[r])) * grad_output[r]).
 #include <atomic>
+#include <mutex>
 #include "bmt_device.h"
 #include "bmt_host.h"
 #include "../../include/bmt_hip.h"
@@ -545,6 +546,116 @@ __global__ __launch_bounds__(kFlatThreads) void ce_flat_vec_kernel(
     }
 }
 
+// ---- the element-wise kernels as a resident grid --------------------------------------------
+// Large arrays with rows of at least 8,192 elements (a multiple of 8, base 16-byte aligned) run the way the
+// long Adam launches do (see adam.hip): one workgroup of 256 lanes per compute unit stays resident and works
+// through tiles of 1,024 vectors (16 KiB = four 4 KiB blocks, one load per lane and block) handed out by atomic
+// tickets, with the loads of the next tile in flight while the current one is computed and stored; the vector
+// memory instructions of the loop and their waits are written by hand.  A tile spans at most two rows, so the
+// per-row scalars (grad_output / max, target / sum) of both are fetched with scalar loads, outside the vector
+// memory counter.
+//
+// The array is transformed in place and the call has no output-only memory, so the ticket counters cannot live
+// in a caller's buffer: they live in a small fixed array in the library's device image, one group of eight
+// counters per stream that has been seen on the device (up to kFlatSlots; launches on one stream follow each other,
+// so a group is never shared by two running launches).  Launches on a stream that is being captured into a graph,
+// on the per-thread default stream, or beyond the slot table keep the workgroup-per-tile kernel.
+constexpr int kFlatStreamThreads = 256;
+constexpr int kFlatStreamVecs = 4;                    // vectors per lane and tile
+constexpr int kFlatCounters = 8;
+constexpr int kFlatSlots = 256;
+constexpr int64_t kFlatStreamMinVec = (int64_t)1 << 22;       // 64 MiB
+constexpr int32_t kFlatStreamMinRow = kFlatStreamThreads * kFlatStreamVecs * 8;
+// counter c of slot s: word c * 1024 + s * 4 (the counters of one launch sit 4 KiB apart)
+static __device__ __align__(256) uint32_t flat_tickets[kFlatCounters * 1024];
+
+__global__ void ce_flat_reset_kernel(uint32_t *tickets, uint32_t first_ticket) {
+    if (threadIdx.x < kFlatCounters) tickets[threadIdx.x * 1024] = first_ticket;
+}
+
+template <typename T, int OP>
+__global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
+    int32_t n, int64_t total_vec, int64_t ntiles, u32x4 *__restrict__ xv, const float *__restrict__ row_a,
+    const float *__restrict__ row_b, const int32_t *__restrict__ target, uint32_t *__restrict__ tickets) {
+    constexpr int V = kFlatStreamVecs;
+    constexpr int64_t kTileVecs = (int64_t)kFlatStreamThreads * V;
+    struct Set {
+        u32x4 w[V];
+        int64_t base;        // first vector of the tile
+        float a0, a1, b0, b1;
+        int32_t t0, t1;      // targets of the tile's first row and of the row after it
+        uint32_t col0;       // column of the tile's first element
+        bool real;
+    };
+    __shared__ uint32_t handed[2];
+    const int which = (int)((blockIdx.x >> 3) & (kFlatCounters - 1));
+    const uint32_t q = ((blockIdx.x >> 6) << 3) | (blockIdx.x & 7u);      // number among the workgroups of this counter
+    uint32_t *counter = tickets + which * 1024;
+    const int64_t first = (int64_t)q * kFlatCounters + which;
+    int64_t ahead = (int64_t)(q + (gridDim.x >> 3)) * kFlatCounters + which;
+    if (first >= ntiles) return;
+    uint32_t drawn = 0;
+    if (threadIdx.x == 0) stream_draw(drawn, counter);
+    const uint32_t row_vecs = (uint32_t)n >> 3;
+    const uint32_t last_row = (uint32_t)total_vec / row_vecs - 1;
+
+    auto issue = [&](Set &s, int64_t tile_in) {
+        s.real = tile_in < ntiles;
+        const int64_t tile = s.real ? tile_in : 0;
+        s.base = tile * kTileVecs;
+        const uint32_t row0 = (uint32_t)s.base / row_vecs;       // the launcher keeps total_vec below 2^32
+        s.col0 = 8u * ((uint32_t)s.base - row0 * row_vecs);
+        const uint32_t row1 = row0 == last_row ? row0 : row0 + 1;     // the last row has no successor
+        s.a0 = row_a[row0]; s.a1 = row_a[row1];
+        if (OP == 0) { s.t0 = target[row0]; s.t1 = target[row1]; s.b0 = s.b1 = 0.f; }
+        else { s.b0 = kTwoPowMinusBias / row_b[row0]; s.b1 = kTwoPowMinusBias / row_b[row1]; s.t0 = s.t1 = -1; }
+#pragma unroll
+        for (int u = 0; u < V; u++) {
+            const int64_t g = s.base + u * kFlatStreamThreads + threadIdx.x;
+            stream_load(s.w[u], xv + (s.real && g < total_vec ? g : 0));
+        }
+    };
+    auto finish = [&](Set &s) {
+        if (!s.real) return;
+#pragma unroll
+        for (int u = 0; u < V; u++) {
+            const int64_t g = s.base + u * kFlatStreamThreads + threadIdx.x;
+            if (g >= total_vec) continue;
+            const uint32_t off = s.col0 + 8u * (uint32_t)(u * kFlatStreamThreads + threadIdx.x);
+            const bool next_row = off >= (uint32_t)n;
+            const int32_t col = (int32_t)(next_row ? off - (uint32_t)n : off);
+            const float a = next_row ? s.a1 : s.a0, b = next_row ? s.b1 : s.b0;
+            const int32_t tk = OP == 0 ? (next_row ? s.t1 : s.t0) - col : -1;
+            u32x4 o;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const float lo = flat_elem<T, OP>(lo_f32<T>(s.w[u][k]), tk == 2 * k, a, b);
+                const float hi = flat_elem<T, OP>(hi_f32<T>(s.w[u][k]), tk == 2 * k + 1, a, b);
+                o[k] = pack2<T>(lo, hi);
+            }
+            stream_store(xv + g, o);
+        }
+    };
+    auto stage = [&](Set &cur, Set &next, int slot) -> int64_t {
+        const int64_t tile = ahead;
+        issue(next, tile);
+        asm volatile("s_waitcnt vmcnt(4)" : "+v"(cur.w[0]), "+v"(cur.w[1]), "+v"(cur.w[2]), "+v"(cur.w[3]), "+v"(drawn));
+        if (threadIdx.x == 0) handed[slot] = drawn;
+        __syncthreads();
+        ahead = (int64_t)handed[slot] * kFlatCounters + which;
+        if (threadIdx.x == 0) stream_draw(drawn, counter);
+        finish(cur);
+        return tile;
+    };
+    Set a, b;
+    issue(a, first);
+    while (true) {
+        if (stage(a, b, 0) >= ntiles) break;
+        if (stage(b, a, 1) >= ntiles) break;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+}
+
 template <typename T, int OP>
 __global__ __launch_bounds__(kFlatScalarThreads) void ce_flat_scalar_kernel(
     int32_t n, int64_t total, uint16_t *__restrict__ x, const float *__restrict__ row_a,
@@ -671,6 +782,36 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
     return e == hipSuccess ? 0 : fail((int)e, who, e);
 }
 
+// The ticket counters of the resident element-wise kernel for `stream` on the current device, or null when the
+// launch has to use the workgroup-per-tile kernel (see ce_flat_stream_kernel).
+static uint32_t *flat_tickets_for(hipStream_t stream) {
+    struct PerDevice { uint32_t *base = nullptr; hipStream_t streams[kFlatSlots]; int used = 0; };
+    static std::mutex mu;
+    static PerDevice devices[64];
+    if (stream == hipStreamPerThread) return nullptr;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    PerDevice &d = devices[dev];
+    if (d.base == nullptr && hipGetSymbolAddress((void **)&d.base, HIP_SYMBOL(flat_tickets)) != hipSuccess) {
+        (void)hipGetLastError();
+        d.base = nullptr;
+        return nullptr;
+    }
+    int slot = 0;
+    while (slot < d.used && d.streams[slot] != stream) slot++;
+    if (slot == d.used) {
+        if (d.used == kFlatSlots) return nullptr;
+        d.streams[d.used++] = stream;
+    }
+    return d.base + slot * 4;
+}
+
 template <typename T, int OP>
 static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void *row_b, const void *target, void *stream,
                    const char *who) {
@@ -686,6 +827,19 @@ static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void 
         int64_t tiles = (total_vec + kFlatThreads * kFlatUnroll - 1) / (kFlatThreads * kFlatUnroll);
         if (tiles < 1) tiles = 1;
         if (tiles > 0x7FFFFFFF) return fail(-1, "cross_entropy launcher: tensor too large for one launch");
+        if (n % 8 == 0 && head == 0 && n >= kFlatStreamMinRow && total_vec >= kFlatStreamMinVec && total_vec < ((int64_t)1 << 32)) {
+            if (uint32_t *tickets = flat_tickets_for(s)) {
+                const int cus = device_cu_count();
+                const unsigned grid = (unsigned)(cus >= 64 ? cus / 64 * 64 : 64);      // 8 XCDs x 8 counters
+                const int64_t per_tile = (int64_t)kFlatStreamThreads * kFlatStreamVecs;
+                hipLaunchKernelGGL(ce_flat_reset_kernel, dim3(1), dim3(64), 0, s, tickets, 2 * (grid / kFlatCounters));
+                hipLaunchKernelGGL((ce_flat_stream_kernel<T, OP>), dim3(grid), dim3(kFlatStreamThreads), 0, s, n, total_vec,
+                                   (total_vec + per_tile - 1) / per_tile, (u32x4 *)x, (const float *)row_a, (const float *)row_b,
+                                   (const int32_t *)target, tickets);
+                hipError_t e = hipGetLastError();
+                return e == hipSuccess ? 0 : fail((int)e, who, e);
+            }
+        }
         auto kern = (n % 8 == 0 && head == 0) ? ce_flat_vec_kernel<T, OP, false> : ce_flat_vec_kernel<T, OP, true>;
         hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(kFlatThreads), 0, s, n, (int32_t)head, total_vec, total,
                            (uint16_t *)x, (const float *)row_a, (const float *)row_b, (const int32_t *)target);

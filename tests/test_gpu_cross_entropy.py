@@ -209,6 +209,49 @@ def test_sumexp_and_softmax_inplace(name, dtype):
         assert ulp_distance16(bits16(xg), want).max() <= 1
 
 
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_elementwise_kernels_on_a_large_array(name, dtype):
+    """Arrays of 2^25 elements or more with rows of 8,192 or more run as a resident grid whose tiles (8,192
+    elements) straddle rows and whose last tile is ragged: 1,049 rows of 32,008.  Backward is bit-exact on identical
+    input, the in-place softmax within one unit in the last place; two launches on two streams at once use separate
+    ticket counters; the words behind the array stay as they were."""
+    m, n = 1049, 32008
+    assert m * n >= 1 << 25 and (m * n // 8) % 1024 != 0 and n % 8192 != 0
+    x, t = _case(m, n, dtype, seed=77)
+    soft, _ = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
+    v = (torch.rand(m, generator=torch.Generator().manual_seed(5)) * 32768.0 / m).float()
+    v[t == -100] = 0
+    want = soft.copy()
+    oracle.ce_backward_inplace(v.numpy(), t.numpy(), want, -100, name)
+    guard = 4096
+    side = torch.cuda.Stream()
+    bufs = []
+    for _ in range(2):
+        buf = torch.full((m * n + guard,), 1.0, dtype=dtype, device="cuda")
+        buf[:m * n].view(m, n).copy_(from_bits16(soft, dtype).reshape(m, n))
+        bufs.append(buf)
+    vg, tg = v.cuda(), t.cuda()
+    torch.cuda.synchronize()
+    F.cross_entropy_backward_inplace(m, n, vg, tg, bufs[0][:m * n].view(m, n), -100)
+    with torch.cuda.stream(side):
+        F.cross_entropy_backward_inplace(m, n, vg, tg, bufs[1][:m * n].view(m, n), -100)
+    torch.cuda.synchronize()
+    for buf in bufs:
+        assert np.array_equal(bits16(buf[:m * n]).reshape(m, n), want)
+        assert bool((buf[m * n:] == 1.0).all())
+
+    buf = bufs[0]
+    xg = buf[:m * n].view(m, n)
+    xg.copy_(x)
+    mx = xg.float().max(-1).values.contiguous()
+    want_se = oracle.fused_sumexp(bits16(x), mx.cpu().numpy(), name)
+    want = bits16(x)
+    oracle.fused_softmax_inplace(want, mx.cpu().numpy(), want_se, name)
+    F.fused_softmax_inplace(xg, mx, torch.from_numpy(want_se).cuda())
+    assert ulp_distance16(bits16(xg), want).max() <= 1
+    assert bool((buf[m * n:] == 1.0).all())
+
+
 # ---- module level, shaped like the reference's tests/test_loss_func.py -----------------------
 def _run(x, tgt, loss_func, scale=32768, use_float=False):
     x = x.clone().detach()
