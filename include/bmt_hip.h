@@ -52,8 +52,10 @@ BMT_API int has_nan_inf_bf16_launcher(int64_t n, const void *g_bf16, void *mid, 
  * One fused step over n elements.  fp16 flavour: g is the loss-scaled gradient and
  * the moments are kept multiplied by `scale` (m in fp16, v in fp32).
  * Writes param_fp32, param_fp16 (round-to-nearest-even), m_fp16, v_fp32.  n <= 0: no-op.
- * param_fp16 is output only: while a launch of 2^25 elements or more is in flight its last
- * 8 bytes hold a tile counter, and its previous contents are never read.
+ * param_fp16 is output only and its previous contents are never read: while a launch of 2^24
+ * elements or more is in flight, four of its last 1,537 8-byte groups hold tile counters (set by a
+ * small kernel in front, replaced by the real values by one behind, in stream order).  A call whose
+ * param_fp16 overlaps g_fp16, param_fp32, m_fp16 or v_fp32 returns -1, at any size.
  */
 BMT_API int adam_fp16_launcher(int64_t n, void *param_fp32, void *param_fp16, const void *g_fp16,
                        void *m_fp16, void *v_fp32,
@@ -149,8 +151,9 @@ BMT_API int fused_softmax_inplace_bf16_launcher(int32_t m, int32_t n, void *logi
  * `count` tensors that share their hyper-parameters (same group, same step count) in as few launches as
  * possible; per element the arithmetic is that of adam_{fp16,bf16}_launcher, bit for bit.
  * `tensors` is a host array; `m` is float[n] for bf16 and half[n] for fp16.  Entries with n <= 0 are skipped.
- * param_16 is output only; a launch over 2^25 elements or more keeps a tile counter in 4 bytes of the
- * last tensor's param_16 while it runs.
+ * param_16 is output only; a launch over 2^24 elements or more keeps four tile counters in the
+ * param_16 of its largest tensor while it runs (as adam_fp16_launcher does), and returns -1 if a param_16
+ * overlaps an input of the same tensor.
  */
 typedef struct bmt_adam_tensor {
     void *param_fp32;
