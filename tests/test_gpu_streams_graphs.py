@@ -94,3 +94,33 @@ def test_step_captured_in_a_graph_replays_like_eager(n):
     graph.replay()
     torch.cuda.synchronize()
     assert flag_g.item() == 1
+
+
+def test_large_in_place_cross_entropy_kernels_captured_in_a_graph():
+    """On a capturing stream the element-wise cross-entropy kernels of large arrays do without the library's ticket
+    counters (a graph may be replayed on any stream, also on two at once); eager launches and replays give the same
+    bits, replay after replay, with eager launches between them."""
+    rows, classes = 1049, 32008                         # 2^25 elements or more: the resident grid when launched eagerly
+    x, t, soft, loss, go = _ce_inputs(rows, classes, 9)
+    LF.cross_entropy_forward(rows, classes, x, t, soft, loss, -100)
+    eager = soft.clone()
+    LF.cross_entropy_backward_inplace(rows, classes, go, t, eager, -100)
+    work = soft.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        LF.cross_entropy_backward_inplace(rows, classes, go, t, work, -100)        # warm-up outside the capture
+        side.synchronize()
+        work.copy_(soft)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            LF.cross_entropy_backward_inplace(rows, classes, go, t, work, -100)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        work.copy_(soft)
+        again = soft.clone()
+        LF.cross_entropy_backward_inplace(rows, classes, go, t, again, -100)        # eager, same counters as before
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(work.view(torch.int16), eager.view(torch.int16))
+        assert torch.equal(again.view(torch.int16), eager.view(torch.int16))
