@@ -252,6 +252,46 @@ def test_elementwise_kernels_on_a_large_array(name, dtype):
     assert bool((buf[m * n:] == 1.0).all())
 
 
+def test_elementwise_kernels_on_more_streams_than_the_library_keeps_counters_for():
+    """The resident grid keeps its ticket counters per stream, for up to 256 streams of a device; launches on further
+    streams take the kernel that needs none.  260 streams, one launch each, same bits everywhere."""
+    m, n = 1049, 32008
+    x, t = _case(m, n, torch.bfloat16, seed=78)
+    soft, _ = oracle.ce_forward(bits16(x), t.numpy(), -100, "bf16")
+    v = torch.full((m,), 1.0 / m)
+    want = soft.copy()
+    oracle.ce_backward_inplace(v.numpy(), t.numpy(), want, -100, "bf16")
+    start = from_bits16(soft, torch.bfloat16).reshape(m, n).cuda()
+    vg, tg = v.cuda(), t.cuda()
+    work = torch.empty_like(start)
+    # torch hands out streams from a pool of 32, so the streams are created through the runtime itself
+    # (looked up through the library under test, so that it is the runtime instance the library and torch share)
+    import ctypes
+    from bmtrain_amd import C
+    hip = C._lib
+    hip.hipStreamCreate.argtypes, hip.hipStreamCreate.restype = [ctypes.POINTER(ctypes.c_void_p)], ctypes.c_int
+    hip.hipStreamDestroy.argtypes, hip.hipStreamDestroy.restype = [ctypes.c_void_p], ctypes.c_int
+    handles = []
+    try:
+        for _ in range(260):
+            handle = ctypes.c_void_p()
+            assert hip.hipStreamCreate(ctypes.byref(handle)) == 0
+            handles.append(handle)
+        torch.cuda.synchronize()
+        for i, handle in enumerate(handles):
+            stream = torch.cuda.ExternalStream(handle.value)
+            with torch.cuda.stream(stream):
+                work.copy_(start, non_blocking=True)
+                F.cross_entropy_backward_inplace(m, n, vg, tg, work, -100)
+            stream.synchronize()
+            if i in (0, 1, 254, 255, 256, 257, 259):
+                assert np.array_equal(bits16(work).reshape(m, n), want), i
+    finally:
+        torch.cuda.synchronize()
+        for handle in handles:
+            hip.hipStreamDestroy(handle)
+
+
 # ---- module level, shaped like the reference's tests/test_loss_func.py -----------------------
 def _run(x, tgt, loss_func, scale=32768, use_float=False):
     x = x.clone().detach()
