@@ -92,6 +92,19 @@ def grad_stats_workspace_floats(n: int) -> int:
     return int(_lib.grad_stats_workspace_floats(n))
 
 
+_lib.bmt_hip_flat_stream_stats.restype = ctypes.c_int
+_lib.bmt_hip_flat_stream_stats.argtypes = [ctypes.POINTER(_i64)]
+
+
+def bmt_hip_flat_stream_stats() -> dict:
+    """Diagnostics of the in-place cross-entropy kernels on the current device: launches that ran as the resident
+    grid, large launches that fell back to the workgroup-per-tile kernel, stream-table entries reassigned."""
+    out = (_i64 * 3)()
+    if _lib.bmt_hip_flat_stream_stats(out) != 0:
+        raise RuntimeError(f"bmt_hip_flat_stream_stats failed: {last_error()}")
+    return {"resident": int(out[0]), "fallback": int(out[1]), "evictions": int(out[2])}
+
+
 class AdamTensor(ctypes.Structure):
     """`bmt_adam_tensor` of include/bmt_hip.h."""
     _fields_ = [("param_fp32", _p), ("param_16", _p), ("grad_16", _p), ("m", _p), ("v", _p), ("n", _i64)]
@@ -122,5 +135,6 @@ adam_bf16_multi_clip_launcher = _bind_multi("adam_bf16_multi_clip_launcher", 1)
 adam_fp16_multi_clip_launcher = _bind_multi("adam_fp16_multi_clip_launcher", 1)
 
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["is_bf16_supported", "bmt_hip_last_error", "grad_stats_workspace_floats",
+                                                  "bmt_hip_flat_stream_stats",
                                                   "adam_bf16_multi_launcher", "adam_fp16_multi_launcher",
                                                   "adam_bf16_multi_clip_launcher", "adam_fp16_multi_clip_launcher"])

@@ -171,7 +171,7 @@ __global__ __launch_bounds__(kAdamThreads) void adam_fp16_vec_kernel(
 }
 
 // ---- long launches: a resident grid that streams ---------------------------------------------
-// From kStreamMinVec 4-element groups on, the step runs as one workgroup of 256 lanes per compute
+// From kStreamMinVecBf16 / kStreamMinVecFp16 4-element groups on, the step runs as one workgroup of 256 lanes per compute
 // unit that stays resident and works through tiles of 256 groups (4 KiB of each fp32 array, the
 // granularity at which HBM channels interleave; tiles of other sizes measured up to 15 points
 // slower).  What decides the rate of this 1:1 read/write stream is how narrow the window of
@@ -208,7 +208,13 @@ __global__ __launch_bounds__(kAdamThreads) void adam_fp16_vec_kernel(
 constexpr int kStreamThreads = 256;
 constexpr int kStreamCounters = 4;
 constexpr int64_t kStreamCounterStride = 512;            // in 8-byte vectors: 4 KiB
-constexpr int64_t kStreamMinVec = (int64_t)1 << 22;      // 2^24 elements
+// Smallest launch (in 4-element groups) that runs as the resident grid, where it overtakes one workgroup per
+// tile (two more one-workgroup launches per call, about 9 us).  Measured per flavour, launches back to back:
+//   bf16   10.5 M elements: 71 % of peak either way;  12.6 M: 74.3 against 71.7;  14.7 M: 76.2 against 73.9;
+//          8.4 M: 70.3 against 74.0;  4.2 M: 58.7 against 70.7
+//   fp16   12.6 M: 70.2 against 73.2;  16.8 M: 73.2 against 73.9;  202 M: 80.0 against 72.8
+constexpr int64_t kStreamMinVecBf16 = (int64_t)3 << 20;   // 12,582,912 elements
+constexpr int64_t kStreamMinVecFp16 = (int64_t)1 << 22;   // 16,777,216 elements
 
 __device__ __forceinline__ bool holds_stream_counter(int64_t i, int64_t nvec) {
     const int64_t d = nvec - 1 - i;
@@ -417,7 +423,7 @@ static hipError_t launch_bf16(int64_t n, float *p32, uint16_t *p16, const uint16
         n, vectorisable, head, nvec,
         [&](unsigned grid) {
             u32x2 *out16 = (u32x2 *)(p16 + head);
-            if (nvec >= kStreamMinVec) {
+            if (nvec >= kStreamMinVecBf16) {
                 const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
                 hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec, stream_grid() / 2);
                 hipLaunchKernelGGL((adam_stream_kernel<false>), dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
@@ -447,7 +453,7 @@ static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16
         n, vectorisable, head, nvec,
         [&](unsigned grid) {
             u32x2 *out16 = (u32x2 *)(p16 + head);
-            if (nvec >= kStreamMinVec) {
+            if (nvec >= kStreamMinVecFp16) {
                 const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
                 hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec, stream_grid() / 2);
                 hipLaunchKernelGGL((adam_stream_kernel<true>), dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
@@ -674,12 +680,20 @@ template <bool FP16>
 static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamHyper &h, hipStream_t s, const char *who) {
     if (count <= 0) return 0;
     if (!tensors) return fail(-1, "adam multi launcher: null tensor table");
+    // The whole table is checked before the first launch, so that an error status means nothing was stepped.
+    for (int32_t k = 0; k < count; k++) {
+        const bmt_adam_tensor &t = tensors[k];
+        if (t.n <= 0) continue;
+        if (!t.param_fp32 || !t.param_16 || !t.grad_16 || !t.m || !t.v) return fail(-1, "adam multi launcher: null pointer");
+        if (output16_overlaps_input(t.n, t.param_16, t.param_fp32, t.grad_16, t.m, FP16 ? 2 : 4, t.v))
+            return fail(-1, "adam multi launcher: param_16 overlaps an input array");
+    }
     AdamBatch batch;
     auto flush = [&]() -> hipError_t {
         if (batch.count == 0) return hipSuccess;
         const uint32_t tiles = batch.first_tile[batch.count];
-        // Batches of 2^22 groups or more run as the resident grid; the tensor with the most groups (at least
-        // 2^22 / 32 of them, so the four counter places exist) lends its 16-bit output to the counters.
+        // Batches of kStreamMinVec* groups or more run as the resident grid; the tensor with the most groups (at
+        // least 3 * 2^20 / 32 of them, so the four counter places exist) lends its 16-bit output to the counters.
         int64_t groups = 0, most = -1;
         batch.stream_first[0] = 0;
         batch.counter_tensor = 0;
@@ -689,7 +703,23 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
             if (nvec > most) { most = nvec; batch.counter_tensor = c; }
             batch.stream_first[c + 1] = batch.stream_first[c] + (uint32_t)((nvec + kStreamThreads - 1) / kStreamThreads);
         }
-        if (groups >= kStreamMinVec) {
+        // The counters occupy the last kStreamCounters * kStreamCounterStride 8-byte vectors of that output while the
+        // launch runs: no array of any other tensor of the batch may share that memory (a table that names one
+        // tensor twice, say).  Such a batch takes the workgroup-per-tile kernel, which keeps no counters.
+        bool counters_clear = true;
+        {
+            const int ct = batch.counter_tensor;
+            const int64_t span = kStreamCounters * kStreamCounterStride < most ? kStreamCounters * kStreamCounterStride : most;
+            const char *lo = (const char *)batch.p16[ct] + (most - span) * 8;
+            for (int c = 0; c < batch.count && counters_clear; c++) {
+                if (c == ct) continue;
+                const int64_t nc = batch.n[c];
+                counters_clear = !overlaps(lo, span * 8, batch.p32[c], 4 * nc) && !overlaps(lo, span * 8, batch.g16[c], 2 * nc) &&
+                                 !overlaps(lo, span * 8, batch.mom[c], (FP16 ? 2 : 4) * nc) && !overlaps(lo, span * 8, batch.var[c], 4 * nc) &&
+                                 !overlaps(lo, span * 8, batch.p16[c], 2 * nc);
+            }
+        }
+        if (counters_clear && groups >= (FP16 ? kStreamMinVecFp16 : kStreamMinVecBf16)) {
             hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, (u32x2 *)batch.p16[batch.counter_tensor], most,
                                stream_grid() / 2);
             hipLaunchKernelGGL((adam_stream_multi_kernel<FP16>), dim3(stream_grid()), dim3(kStreamThreads), 0, s,
@@ -707,9 +737,6 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
     for (int32_t k = 0; k < count; k++) {
         const bmt_adam_tensor &t = tensors[k];
         if (t.n <= 0) continue;
-        if (!t.param_fp32 || !t.param_16 || !t.grad_16 || !t.m || !t.v) return fail(-1, "adam multi launcher: null pointer");
-        if (output16_overlaps_input(t.n, t.param_16, t.param_fp32, t.grad_16, t.m, FP16 ? 2 : 4, t.v))
-            return fail(-1, "adam multi launcher: param_16 overlaps an input array");
         const bool aligned = (((uintptr_t)t.param_fp32 | (uintptr_t)t.v | (FP16 ? 0 : (uintptr_t)t.m)) & 15u) == 0 &&
                              (((uintptr_t)t.param_16 | (uintptr_t)t.grad_16 | (FP16 ? (uintptr_t)t.m : 0)) & 7u) == 0;
         const int64_t tiles = multi_tiles(t.n);

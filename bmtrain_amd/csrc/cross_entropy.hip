@@ -109,6 +109,17 @@ __device__ __forceinline__ RowSpan row_span(const uint16_t *x, int64_t row, int3
     return sp;
 }
 
+// The row of workgroup b when every XCD is to work on its own run of consecutive rows.  Workgroups are handed to
+// the eight XCDs in turn (b % 8), so XCD k takes the k-th eighth of the rows, in order; the rows past the last
+// multiple of eight keep their index.  This is a choice of order only: every row is still processed exactly once
+// whatever the hardware's placement is.  Measured on rows of 32 to 64 KiB (one workgroup of 1024 lanes reading its
+// row and then writing it): 68-74 % of peak with row = b, 77-79 % with this order; rows of 16 KiB or less lose 2-4
+// points and rows beyond 80 KiB gain or lose about one, so only the 1024-lane register-resident kernels use it.
+__device__ __forceinline__ int64_t xcd_contiguous_row(uint32_t b, uint32_t rows) {
+    const uint32_t whole = rows & ~7u;
+    return b < whole ? (int64_t)(b & 7u) * (whole >> 3) + (b >> 3) : (int64_t)b;
+}
+
 // ---- forward, register-resident row ------------------------------------------
 // One workgroup of THREADS lanes per row; lane t owns vectors t, t+THREADS, ...
 // (CHUNKS of them, 8 elements each).  The 8*CHUNKS exponentials of a lane stay in fp32
@@ -118,7 +129,7 @@ __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
     int32_t n, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
     uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
     __shared__ float slots[2][THREADS / kWave];
-    const int64_t row = blockIdx.x;
+    const int64_t row = THREADS == 1024 ? xcd_contiguous_row(blockIdx.x, gridDim.x) : (int64_t)blockIdx.x;
     const RowSpan sp = row_span(x, row, n);
     const int32_t nvec = sp.nvec;
     const u32x4 *xr = (const u32x4 *)(sp.row + sp.head);
@@ -312,6 +323,12 @@ __global__ __launch_bounds__(kSmallThreads) void ce_forward_small_kernel(
 // lane stay in registers and the next LK in LDS; the remaining ones are dropped.  Sweep 2 walks the
 // row backwards: the dropped vectors — the most recently fetched, so the likeliest to sit in L2
 // still — are loaded again, then the LDS and register parts follow without memory traffic.
+// Cache policy decides what that second fetch costs: the first fetch of the dropped part uses the default
+// policy so that the lines stay in L2 and the memory-side cache (fetched non-temporally, the second fetch
+// comes from HBM and the kernel takes 0.92 ms instead of 0.76 at 8,192 x 128,256; each pair of chunks fetched
+// that way costs 0.02-0.05 ms), and the second fetch is non-temporal — its lines are dead afterwards —
+// which gains 1.2 %.  With the first fetch cached, the second one is free: a timing probe that skips it
+// altogether runs no faster.
 // Fine-grained load/compute interleaving in both sweeps lets the 32 waves of a CU hide each
 // other's latencies, which a whole-row-resident scheme with one or two workgroups per CU cannot.
 template <typename T, int RK, int LK>
@@ -376,7 +393,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
 #pragma unroll
         for (int g = 0; g < GROUP; g++) staged[(c0 + g - RK) * THREADS + tid] = v[g];
     }
-    // dropped part: default cache policy, meant to be found in L2 again
+    // dropped part: default cache policy, so that the second fetch finds it in L2 or the memory-side cache
 #pragma unroll 1
     for (int c0 = RK + LK; c0 < chunks; c0 += GROUP) {
         u32x4 v[GROUP];
@@ -403,14 +420,14 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
         srow[i] = T::from_f32(quotient(exp_biased(T::to_f32(sp.row[i]), M), rs));
     }
 
-    // dropped part, last fetched first
+    // dropped part, last fetched first; its lines are not needed again (non-temporal)
 #pragma unroll 1
     for (int c0 = chunks - GROUP; c0 >= RK + LK; c0 -= GROUP) {
         u32x4 v[GROUP];
 #pragma unroll
         for (int g = GROUP - 1; g >= 0; g--) {
             const int j = (c0 + g) * THREADS + tid;
-            v[g] = j < nvec ? xr[j] : pad4;
+            v[g] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
         }
 #pragma unroll
         for (int g = GROUP - 1; g >= 0; g--) {
@@ -601,7 +618,9 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
 
     auto issue = [&](Set &s, int64_t tile_in) {
         s.real = tile_in < ntiles;
-        const int64_t tile = s.real ? tile_in : 0;
+        // the tile number is the same in every lane (it came through LDS): saying so puts the row arithmetic and the
+        // loads of the per-row scalars below on the scalar unit, outside the vector memory counter
+        const int64_t tile = s.real ? (int64_t)__builtin_amdgcn_readfirstlane((uint32_t)tile_in) : 0;
         s.base = tile * kTileVecs;
         const uint32_t row0 = (uint32_t)s.base / row_vecs;       // the launcher keeps total_vec below 2^32
         s.col0 = 8u * ((uint32_t)s.base - row0 * row_vecs);
@@ -782,34 +801,91 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
     return e == hipSuccess ? 0 : fail((int)e, who, e);
 }
 
-// The ticket counters of the resident element-wise kernel for `stream` on the current device, or null when the
-// launch has to use the workgroup-per-tile kernel (see ce_flat_stream_kernel).
-static uint32_t *flat_tickets_for(hipStream_t stream) {
-    struct PerDevice { uint32_t *base = nullptr; hipStream_t streams[kFlatSlots]; int used = 0; };
-    static std::mutex mu;
-    static PerDevice devices[64];
-    if (stream == hipStreamPerThread) return nullptr;
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
-        (void)hipGetLastError();
-        return nullptr;
-    }
+// The ticket counters of the resident element-wise kernel for `stream`, or null when the launch has to use the
+// workgroup-per-tile kernel (see ce_flat_stream_kernel): a stream under graph capture, the per-thread default stream,
+// a stream that belongs to another device than the current one, or a full table with nothing to evict.
+//
+// Every device keeps a table of up to kFlatSlots stream handles; a stream's slot is its group of eight counters.
+// Behind every launch that uses a slot the library records an event of its own on the caller's stream
+// (flat_launch_recorded).  When the table is full, the least recently used slot whose event has completed — so no
+// launch that draws from its counters can still be running, whether or not its stream still exists — is given to
+// the new stream; handles of streams that may have been destroyed are never passed to the runtime.  A process that
+// creates and destroys streams therefore keeps the resident kernel for good.
+struct FlatStreamStats { int64_t resident = 0, fallback = 0, evictions = 0; };
+static FlatStreamStats flat_stats[64];
+static std::mutex flat_mutex;
+struct FlatSlot { hipStream_t stream; uint64_t last_use; hipEvent_t done; bool recorded; };
+struct FlatDevice { uint32_t *base = nullptr; FlatSlot slots[kFlatSlots]; int used = 0; uint64_t clock = 0; };
+static FlatDevice flat_devices[64];
+
+static uint32_t *flat_tickets_for(hipStream_t stream, int *dev_out, int *slot_out) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
-    std::lock_guard<std::mutex> lock(mu);
-    PerDevice &d = devices[dev];
+    auto fallback = [&]() -> uint32_t * {
+        (void)hipGetLastError();
+        std::lock_guard<std::mutex> lock(flat_mutex);
+        flat_stats[dev].fallback++;
+        return nullptr;
+    };
+    if (stream == hipStreamPerThread) return fallback();
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) return fallback();
+    hipDevice_t owner = -1;
+    if (hipStreamGetDevice(stream, &owner) != hipSuccess || (int)owner != dev) return fallback();   // counters are per device
+    std::lock_guard<std::mutex> lock(flat_mutex);
+    FlatDevice &d = flat_devices[dev];
     if (d.base == nullptr && hipGetSymbolAddress((void **)&d.base, HIP_SYMBOL(flat_tickets)) != hipSuccess) {
         (void)hipGetLastError();
         d.base = nullptr;
+        flat_stats[dev].fallback++;
         return nullptr;
     }
     int slot = 0;
-    while (slot < d.used && d.streams[slot] != stream) slot++;
+    while (slot < d.used && d.slots[slot].stream != stream) slot++;
     if (slot == d.used) {
-        if (d.used == kFlatSlots) return nullptr;
-        d.streams[d.used++] = stream;
+        if (d.used < kFlatSlots) {
+            hipEvent_t ev = nullptr;
+            if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+                (void)hipGetLastError();
+                flat_stats[dev].fallback++;
+                return nullptr;
+            }
+            d.slots[slot] = FlatSlot{stream, 0, ev, false};
+            d.used++;
+        } else {
+            // least recently used first; a few event queries at most
+            slot = -1;
+            uint64_t tried_up_to = 0;
+            for (int attempt = 0; attempt < 8 && slot < 0; attempt++) {
+                int oldest = -1;
+                for (int k = 0; k < kFlatSlots; k++)
+                    if (d.slots[k].last_use > tried_up_to && (oldest < 0 || d.slots[k].last_use < d.slots[oldest].last_use)) oldest = k;
+                if (oldest < 0) break;
+                tried_up_to = d.slots[oldest].last_use;
+                if (!d.slots[oldest].recorded) continue;                 // a launch whose end nothing marks: never handed on
+                if (hipEventQuery(d.slots[oldest].done) == hipSuccess) slot = oldest;
+                else (void)hipGetLastError();
+            }
+            if (slot < 0) { flat_stats[dev].fallback++; return nullptr; }
+            flat_stats[dev].evictions++;
+            d.slots[slot].stream = stream;
+        }
     }
+    d.slots[slot].last_use = ++d.clock;
+    d.slots[slot].recorded = false;             // until flat_launch_recorded has marked the end of the launch to come
+    flat_stats[dev].resident++;
+    *dev_out = dev;
+    *slot_out = slot;
     return d.base + slot * 4;
+}
+
+// Marks the end of the launch that was just issued with the counters of `slot` (see flat_tickets_for).
+static void flat_launch_recorded(int dev, int slot, hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(flat_mutex);
+    FlatSlot &sl = flat_devices[dev].slots[slot];
+    if (sl.stream != stream) return;                                     // handed on in between: cannot happen while `recorded` is false
+    if (hipEventRecord(sl.done, stream) == hipSuccess) sl.recorded = true;
+    else (void)hipGetLastError();
 }
 
 template <typename T, int OP>
@@ -828,7 +904,8 @@ static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void 
         if (tiles < 1) tiles = 1;
         if (tiles > 0x7FFFFFFF) return fail(-1, "cross_entropy launcher: tensor too large for one launch");
         if (n % 8 == 0 && head == 0 && n >= kFlatStreamMinRow && total_vec >= kFlatStreamMinVec && total_vec < ((int64_t)1 << 32)) {
-            if (uint32_t *tickets = flat_tickets_for(s)) {
+            int dev = 0, slot = 0;
+            if (uint32_t *tickets = flat_tickets_for(s, &dev, &slot)) {
                 const int cus = device_cu_count();
                 const unsigned grid = (unsigned)(cus >= 64 ? cus / 64 * 64 : 64);      // 8 XCDs x 8 counters
                 const int64_t per_tile = (int64_t)kFlatStreamThreads * kFlatStreamVecs;
@@ -837,6 +914,7 @@ static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void 
                                    (total_vec + per_tile - 1) / per_tile, (u32x4 *)x, (const float *)row_a, (const float *)row_b,
                                    (const int32_t *)target, tickets);
                 hipError_t e = hipGetLastError();
+                flat_launch_recorded(dev, slot, s);
                 return e == hipSuccess ? 0 : fail((int)e, who, e);
             }
         }
@@ -872,6 +950,17 @@ static int sumexp(int32_t m, int32_t n, const void *logits, const void *row_max,
 }  // namespace bmt
 
 using namespace bmt;
+
+extern "C" int bmt_hip_flat_stream_stats(int64_t *out) {
+    if (!out) return fail(-1, "bmt_hip_flat_stream_stats: null pointer");
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(-1, "bmt_hip_flat_stream_stats: no current device");
+    std::lock_guard<std::mutex> lock(flat_mutex);
+    out[0] = flat_stats[dev].resident;
+    out[1] = flat_stats[dev].fallback;
+    out[2] = flat_stats[dev].evictions;
+    return 0;
+}
 
 extern "C" int cross_entropy_forward_fp16_launcher(int32_t m, int32_t n, const void *input, const void *target,
                                                    void *softmax, void *output, int32_t ignore_index, void *stream) {

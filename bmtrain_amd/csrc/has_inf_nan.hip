@@ -205,10 +205,17 @@ constexpr int64_t kStaticPartials = (int64_t)1 << 20;                     // 4 M
 static __device__ __align__(256) float stats_scratch[kStaticPartials];
 static std::atomic<float *> stats_scratch_ptr[64];                         // per device, null until looked up
 
-static float *static_partials(const char **why) {
+static float *static_partials(hipStream_t stream, const char **why) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= 64) { *why = "grad_stats_noalloc_launcher: no current device"; return nullptr; }
+    // the array used is the current device's copy: a stream of another device would run the kernels over there
+    hipDevice_t owner = -1;
+    if (stream != hipStreamPerThread && (hipStreamGetDevice(stream, &owner) != hipSuccess || (int)owner != dev)) {
+        (void)hipGetLastError();
+        *why = "grad_stats_noalloc_launcher: the stream does not belong to the current device";
+        return nullptr;
+    }
     float *ptr = stats_scratch_ptr[dev].load(std::memory_order_acquire);
     if (ptr == nullptr) {
         e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(stats_scratch));
@@ -225,7 +232,7 @@ extern "C" int grad_stats_noalloc_launcher(int64_t n, const void *g_16, int32_t 
     if (bmt::stats_tiles(n, g_16, nullptr, nullptr) > bmt::kStaticPartials)
         return bmt::fail(-1, "grad_stats_noalloc_launcher: more than 2^36 elements; use grad_stats_*_launcher with a workspace");
     const char *why = "";
-    float *partials = bmt::static_partials(&why);
+    float *partials = bmt::static_partials((hipStream_t)stream, &why);
     if (partials == nullptr) return bmt::fail(-1, why);
     return is_bf16 ? bmt::grad_stats<bmt::BFloat16>(n, g_16, sumsq, flag, partials, stream, "grad_stats_noalloc_launcher")
                    : bmt::grad_stats<bmt::Half>(n, g_16, sumsq, flag, partials, stream, "grad_stats_noalloc_launcher");

@@ -14,11 +14,25 @@
  *     never looks at the launch status.  bmt_hip_last_error() describes the last
  *     failure of the calling thread.
  *
- * Ownership: the caller owns every buffer; the library allocates no device memory,
- * retains no pointer and keeps no state between calls apart from the host Adam's
- * parked worker threads.  GPU launchers are asynchronous
- * on `stream` (a hipStream_t; NULL = the default stream) and never synchronise.
- * Device pointers must belong to the device that is current at the call.
+ * Ownership: the caller owns every buffer; the library allocates no device memory
+ * and retains no pointer into a caller's buffer.  GPU launchers are asynchronous on
+ * `stream` (a hipStream_t; NULL = the default stream) and never synchronise.
+ * Device pointers and the stream must belong to the device that is current at the call.
+ *
+ * State the library does keep (everything else is stateless, as the reference's launchers are):
+ *   - host side: the parked worker threads of adam_cpu_*_launcher; per device, a table of up to 256
+ *     stream handles (which stream uses which group of ticket counters below) with one event each, behind one mutex, the
+ *     looked-up addresses of the two device arrays, and the cached compute-unit count;
+ *   - device side, two fixed arrays in the library's own code object, one copy per GPU: 32 KiB of
+ *     ticket counters for the in-place cross-entropy kernels (eight counters per stream in the table)
+ *     and the 4 MiB of partial sums of grad_stats_noalloc_launcher;
+ *   - in a caller's buffer, only for the duration of a launch: long Adam launches keep four tile
+ *     counters in the 16-bit parameter output (see adam_fp16_launcher).
+ * The library records one event of its own on the caller's stream behind every launch that uses a table
+ * entry.  When the table is full, the least recently used entry whose event has completed is given to the
+ * new stream; if the entries looked at are all busy the launch runs the kernel that needs no counters
+ * (same results, a few per cent slower).  Launches on a stream under
+ * graph capture, on hipStreamPerThread or on a stream of another device always take that kernel.
  */
 #ifndef BMT_HIP_H
 #define BMT_HIP_H
@@ -53,7 +67,7 @@ BMT_API int has_nan_inf_bf16_launcher(int64_t n, const void *g_bf16, void *mid, 
  * the moments are kept multiplied by `scale` (m in fp16, v in fp32).
  * Writes param_fp32, param_fp16 (round-to-nearest-even), m_fp16, v_fp32.  n <= 0: no-op.
  * param_fp16 is output only and its previous contents are never read: while a launch of 2^24
- * elements or more is in flight, four of its last 1,537 8-byte groups hold tile counters (set by a
+ * elements or more (bf16 flavour: 12,582,912 or more) is in flight, four of its last 1,537 8-byte groups hold tile counters (set by a
  * small kernel in front, replaced by the real values by one behind, in stream order).  A call whose
  * param_fp16 overlaps g_fp16, param_fp32, m_fp16 or v_fp32 returns -1, at any size.
  */
@@ -211,6 +225,15 @@ BMT_API int grad_stats_bf16_launcher(int64_t n, const void *g_bf16, void *sumsq,
  */
 BMT_API int grad_stats_noalloc_launcher(int64_t n, const void *g_16, int32_t is_bf16, void *sumsq, void *flag,
                                         void *stream);
+
+/*
+ * bmt_hip_flat_stream_stats — diagnostics, no counterpart in the reference.  For the current device, since the
+ * library was loaded: out[0] = launches of the in-place cross-entropy / softmax kernels that ran as the resident
+ * ticket-ordered grid, out[1] = large launches that could not get ticket counters (stream under capture,
+ * hipStreamPerThread, stream of another device, stream table full of busy streams) and took the
+ * workgroup-per-tile kernel, out[2] = stream-table entries handed from one stream to another.
+ */
+BMT_API int bmt_hip_flat_stream_stats(int64_t *out);
 
 #ifdef __cplusplus
 }

@@ -206,6 +206,53 @@ def test_argument_checks():
     F.adam_bf16(p, both[n:], both[:n], m, v, *a)          # adjacent is fine
 
 
+def test_a_bad_entry_anywhere_in_a_multi_tensor_table_means_nothing_was_stepped():
+    """The multi-tensor launcher checks its whole table before the first launch: 70 tensors (three launches' worth)
+    with the last one's 16-bit output overlapping its gradient are refused, and no tensor — not even those of the
+    first two launches — has been touched."""
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    rows, originals = [], []
+    for k in range(70):
+        n = 5000 + 4 * k
+        p = torch.randn(n, generator=gen, device="cuda") * 0.02
+        g = (torch.randn(n, generator=gen, device="cuda") * 1e-3).bfloat16()
+        rows.append((p, torch.full((n,), -1, dtype=torch.bfloat16, device="cuda"), g, torch.zeros(n, device="cuda"),
+                     torch.zeros(n, device="cuda")))
+        originals.append(p.clone())
+    p, h, g, m, v = rows[-1]
+    rows[-1] = (p, g.view(torch.bfloat16), g, m, v)              # 16-bit output == gradient
+    with pytest.raises(RuntimeError, match="overlaps"):
+        F.adam_multi(rows, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 3)
+    torch.cuda.synchronize()
+    for (p, h, g, m, v), p0 in zip(rows[:-1], originals):
+        assert torch.equal(p, p0) and torch.count_nonzero(m) == 0 and torch.count_nonzero(v) == 0
+        assert torch.equal(h.view(torch.int16), torch.full_like(h, -1).view(torch.int16))
+
+
+def test_a_long_batch_whose_counter_host_is_shared_takes_the_kernel_without_counters():
+    """A long batch keeps its tile counters in the tail of the largest tensor's 16-bit output.  When another entry
+    of the table shares that memory (here: a second tensor whose 16-bit output is a view into the large tensor's
+    output tail — its values are overwritten by whichever store comes last, as in any table that names memory
+    twice), the batch must not keep counters there: the large tensor's fp32 state, which nothing else touches,
+    comes out exactly as from a launch of its own."""
+    n = (3 << 22) + 4096
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    p = torch.randn(n, generator=gen, device="cuda") * 0.02
+    g = (torch.randn(n, generator=gen, device="cuda") * 1e-3).bfloat16()
+    alone = (p.clone(), torch.zeros(n, dtype=torch.bfloat16, device="cuda"), g, torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda"))
+    F.adam_bf16(*alone, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 3)
+    big = (p.clone(), torch.zeros(n, dtype=torch.bfloat16, device="cuda"), g, torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda"))
+    k = 4096
+    small = (torch.zeros(k, device="cuda"), big[1][n - k:], torch.zeros(k, dtype=torch.bfloat16, device="cuda"),
+             torch.zeros(k, device="cuda"), torch.zeros(k, device="cuda"))
+    F.adam_multi([big, small], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 3)
+    torch.cuda.synchronize()
+    for a, b in zip((alone[0], alone[3], alone[4]), (big[0], big[3], big[4])):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    assert torch.equal(alone[1][:n - k].view(torch.int16), big[1][:n - k].view(torch.int16))
+    assert torch.count_nonzero(small[0]) == 0                     # zero gradient, zero state: the small tensor stays zero
+
+
 def _fill_(x, std, gen, absolute=False, chunk=1 << 27):
     for lo in range(0, x.numel(), chunk):
         part = x[lo:lo + chunk]
@@ -253,13 +300,15 @@ def test_one_transformer_block_flat_buffer():
 
 
 @pytest.mark.parametrize("flavour", ["bf16", "fp16"])
-@pytest.mark.parametrize("n,off", [((1 << 24) - 1, 0), ((1 << 24) + 2, 2), ((1 << 24) + 1024 * 7 + 5, 1), ((1 << 24) + 4 * 2048 + 3, 0),
+@pytest.mark.parametrize("n,off", [((3 << 22) - 1, 0), ((3 << 22) + 2, 2), ((3 << 22) + 1024 * 7 + 5, 1), ((3 << 22) + 12, 3),
+                                   ((1 << 24) - 1, 0), ((1 << 24) + 2, 2), ((1 << 24) + 1024 * 7 + 5, 1), ((1 << 24) + 4 * 2048 + 3, 0),
                                    ((1 << 25) + 12345, 0), ((1 << 25) + 4096 * 3 + 1, 2), (3 * (1 << 24) + 4 * 1537, 3)])
 def test_around_the_launch_size_where_the_resident_grid_takes_over(flavour, n, off):
-    """From 2^22 four-element groups on, a resident grid draws tiles of 256 groups from four counters kept in the
-    16-bit output (word 0 of the vectors nvec-1, nvec-513, nvec-1025, nvec-1537), whose real values a small kernel
-    restores afterwards.  Whole-buffer comparison with the oracle just below and above that size, with unaligned
-    heads and partial last tiles: every tile stepped exactly once, and the counters' places hold their real values."""
+    """From 3 * 2^20 (bf16) or 2^22 (fp16) four-element groups on, a resident grid draws tiles of 256 groups from four
+    counters kept in the 16-bit output (word 0 of the vectors nvec-1, nvec-513, nvec-1025, nvec-1537), whose real
+    values a small kernel restores afterwards.  Whole-buffer comparison with the oracle just below and above both
+    sizes, with unaligned heads and partial last tiles: every tile stepped exactly once, and the counters' places
+    hold their real values."""
     dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
     mdt = torch.float16 if flavour == "fp16" else torch.float32
     scale = 4.0 if flavour == "fp16" else 1.0
@@ -355,7 +404,7 @@ def test_multi_tensor_launch_equals_per_tensor_launches(flavour):
 
 @pytest.mark.parametrize("flavour", ["bf16", "fp16"])
 def test_long_multi_tensor_launch_runs_as_one_resident_grid(flavour):
-    """Batches of 2^24 elements or more run as one resident grid over all their tensors: tiles of 256 groups numbered
+    """Batches of 3 * 2^22 (bf16) or 2^24 (fp16) elements or more run as one resident grid over all their tensors: tiles of 256 groups numbered
     through the tensors, drawn by ticket from four counters kept in the 16-bit output of the largest tensor; leftover
     elements and the counters' places are finished by a small kernel.  40 tensors (two launches, the second a short
     one), 33 equal tensors, and a mix of sizes from 3 to 2^24 + 5 elements with every leftover count — bit for bit
@@ -364,7 +413,9 @@ def test_long_multi_tensor_launch_runs_as_one_resident_grid(flavour):
     mdt = torch.float16 if flavour == "fp16" else torch.float32
     fn = F.adam_fp16 if flavour == "fp16" else F.adam_bf16
     for sizes in ([1_200_001 + 4 * k for k in range(39)] + [2_000_003], [1_200_000] * 32 + [4096 * 300 + 3],
-                  [(1 << 24) + 5, 77, 4096, (1 << 22) + 2, 3, 1_000_001, 255, 1024, 1023, 6, (1 << 23) + 3]):
+                  [(1 << 24) + 5, 77, 4096, (1 << 22) + 2, 3, 1_000_001, 255, 1024, 1023, 6, (1 << 23) + 3],
+                  [(1 << 22) + 1, (1 << 23) + 2, 4099, 255],          # 12.6 M elements: resident for bf16, short kernel for fp16
+                  [(3 << 22) - 8192, 4096, 4097]):                     # just above the bf16 size, the largest tensor just below it
         gen = torch.Generator(device="cuda").manual_seed(len(sizes))
         single, multi = [], []
         for n in sizes:

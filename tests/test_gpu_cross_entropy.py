@@ -253,8 +253,9 @@ def test_elementwise_kernels_on_a_large_array(name, dtype):
 
 
 def test_elementwise_kernels_on_more_streams_than_the_library_keeps_counters_for():
-    """The resident grid keeps its ticket counters per stream, for up to 256 streams of a device; launches on further
-    streams take the kernel that needs none.  260 streams, one launch each, same bits everywhere."""
+    """The resident grid keeps its ticket counters per stream, for up to 256 streams of a device; a launch on a further
+    stream gets the table entry of a stream whose last launch has completed, or takes the kernel that needs no
+    counters.  260 streams, one launch each, same bits everywhere."""
     m, n = 1049, 32008
     x, t = _case(m, n, torch.bfloat16, seed=78)
     soft, _ = oracle.ce_forward(bits16(x), t.numpy(), -100, "bf16")

@@ -124,3 +124,95 @@ def test_large_in_place_cross_entropy_kernels_captured_in_a_graph():
         torch.cuda.synchronize()
         assert torch.equal(work.view(torch.int16), eager.view(torch.int16))
         assert torch.equal(again.view(torch.int16), eager.view(torch.int16))
+
+
+def _runtime():
+    """hipStreamCreate / hipStreamDestroy of the runtime instance the library and torch share (torch itself hands
+    out streams from a pool of 32 and never destroys one)."""
+    import ctypes
+    from bmtrain_amd import C
+    hip = C._lib
+    hip.hipStreamCreate.argtypes, hip.hipStreamCreate.restype = [ctypes.POINTER(ctypes.c_void_p)], ctypes.c_int
+    hip.hipStreamDestroy.argtypes, hip.hipStreamDestroy.restype = [ctypes.c_void_p], ctypes.c_int
+    return hip, ctypes
+
+
+def test_a_process_that_recycles_streams_keeps_the_resident_kernel():
+    """The resident in-place kernel keeps eight ticket counters per stream in a table of 256 streams per device.
+    700 streams are created through the runtime, used for one large in-place launch each and destroyed (300 are alive
+    at any time — the runtime reuses the addresses of destroyed streams, so only streams that are alive together have
+    different handles): every launch must still run as the resident grid — the table entry of a
+    stream whose last launch has completed is handed on — and every checked result equals the first one."""
+    from bmtrain_amd import C
+    hip, ctypes = _runtime()
+    rows, classes = 1049, 32008
+    x, t, soft, loss, go = _ce_inputs(rows, classes, 11)
+    LF.cross_entropy_forward(rows, classes, x, t, soft, loss, -100)
+    expect = soft.clone()
+    LF.cross_entropy_backward_inplace(rows, classes, go, t, expect, -100)
+    torch.cuda.synchronize()
+    before = C.bmt_hip_flat_stream_stats()
+    work = [soft.clone() for _ in range(4)]
+    alive, seen = [], set()
+    try:
+        for k in range(700):
+            handle = ctypes.c_void_p()
+            assert hip.hipStreamCreate(ctypes.byref(handle)) == 0
+            alive.append(handle)
+            seen.add(handle.value)
+            if len(alive) > 300:
+                torch.cuda.synchronize()
+                assert hip.hipStreamDestroy(alive.pop(0)) == 0
+            buf = work[k % 4]
+            side = torch.cuda.ExternalStream(handle.value)
+            with torch.cuda.stream(side):
+                buf.copy_(soft, non_blocking=True)
+                LF.cross_entropy_backward_inplace(rows, classes, go, t, buf, -100)
+            side.synchronize()
+            if k % 50 == 49 or k >= 696:
+                assert torch.equal(buf.view(torch.int16), expect.view(torch.int16)), k
+    finally:
+        torch.cuda.synchronize()
+        for handle in alive:
+            hip.hipStreamDestroy(handle)
+    after = C.bmt_hip_flat_stream_stats()
+    assert len(seen) > 256                                # more distinct handles than the table has entries
+    assert after["resident"] - before["resident"] == 700
+    assert after["fallback"] == before["fallback"]
+    assert after["evictions"] - before["evictions"] >= len(seen) - 256
+
+
+def test_entries_of_streams_with_work_in_flight_are_not_handed_on():
+    """300 runtime streams, each with its own buffer, all launched without waiting in between, three rounds: whatever
+    the table does for the streams beyond its 256 entries (hand on an entry whose launch has completed, or take the
+    kernel without counters), no two running launches may share counters — every buffer comes out exact."""
+    from bmtrain_amd import C
+    hip, ctypes = _runtime()
+    rows, classes = 1049, 32008
+    x, t, soft, loss, go = _ce_inputs(rows, classes, 12)
+    LF.cross_entropy_forward(rows, classes, x, t, soft, loss, -100)
+    expect = soft.clone()
+    LF.cross_entropy_backward_inplace(rows, classes, go, t, expect, -100)
+    torch.cuda.synchronize()
+    handles = []
+    try:
+        for _ in range(300):
+            handle = ctypes.c_void_p()
+            assert hip.hipStreamCreate(ctypes.byref(handle)) == 0
+            handles.append(handle)
+        bufs = [torch.empty_like(soft) for _ in handles]
+        before = C.bmt_hip_flat_stream_stats()
+        for rnd in range(3):
+            for handle, buf in zip(handles, bufs):
+                with torch.cuda.stream(torch.cuda.ExternalStream(handle.value)):
+                    buf.copy_(soft, non_blocking=True)
+                    LF.cross_entropy_backward_inplace(rows, classes, go, t, buf, -100)
+            torch.cuda.synchronize()
+            for k, buf in enumerate(bufs):
+                assert torch.equal(buf.view(torch.int16), expect.view(torch.int16)), (rnd, k)
+        after = C.bmt_hip_flat_stream_stats()
+        assert after["resident"] + after["fallback"] - before["resident"] - before["fallback"] == 900
+    finally:
+        torch.cuda.synchronize()
+        for handle in handles:
+            hip.hipStreamDestroy(handle)
