@@ -583,17 +583,28 @@ constexpr int kFlatCounters = 8;
 constexpr int kFlatSlots = 256;
 constexpr int64_t kFlatStreamMinVec = (int64_t)1 << 22;       // 64 MiB
 constexpr int32_t kFlatStreamMinRow = kFlatStreamThreads * kFlatStreamVecs * 8;
-// counter c of slot s: word c * 1024 + s * 4 (the counters of one launch sit 4 KiB apart)
+// counter c of slot s: word c * 1024 + s * 4 (the counters of one launch sit 4 KiB apart); word s * 4 + 1 counts the
+// workgroups of the running launch that have left
 static __device__ __align__(256) uint32_t flat_tickets[kFlatCounters * 1024];
 
 __global__ void ce_flat_reset_kernel(uint32_t *tickets, uint32_t first_ticket) {
     if (threadIdx.x < kFlatCounters) tickets[threadIdx.x * 1024] = first_ticket;
+    if (threadIdx.x == kFlatCounters) tickets[1] = 0u;
+}
+// The last workgroup to leave a launch writes the launch's number into the slot's word of pinned host memory:
+// from then on nothing draws from the slot's counters, and the host may hand the slot to another stream.
+__device__ __forceinline__ void flat_leave(uint32_t *tickets, uint32_t *done_word, uint32_t launch_number) {
+    if (threadIdx.x == 0) {
+        const uint32_t left = __hip_atomic_fetch_add(tickets + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (left + 1 == gridDim.x) __hip_atomic_store(done_word, launch_number, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
 }
 
 template <typename T, int OP>
 __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
     int32_t n, int64_t total_vec, int64_t ntiles, u32x4 *__restrict__ xv, const float *__restrict__ row_a,
-    const float *__restrict__ row_b, const int32_t *__restrict__ target, uint32_t *__restrict__ tickets) {
+    const float *__restrict__ row_b, const int32_t *__restrict__ target, uint32_t *__restrict__ tickets,
+    uint32_t *__restrict__ done_word, uint32_t launch_number) {
     constexpr int V = kFlatStreamVecs;
     constexpr int64_t kTileVecs = (int64_t)kFlatStreamThreads * V;
     struct Set {
@@ -610,7 +621,7 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
     uint32_t *counter = tickets + which * 1024;
     const int64_t first = (int64_t)q * kFlatCounters + which;
     int64_t ahead = (int64_t)(q + (gridDim.x >> 3)) * kFlatCounters + which;
-    if (first >= ntiles) return;
+    if (first >= ntiles) { flat_leave(tickets, done_word, launch_number); return; }
     uint32_t drawn = 0;
     if (threadIdx.x == 0) stream_draw(drawn, counter);
     const uint32_t row_vecs = (uint32_t)n >> 3;
@@ -673,6 +684,7 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
         if (stage(b, a, 1) >= ntiles) break;
     }
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+    flat_leave(tickets, done_word, launch_number);
 }
 
 template <typename T, int OP>
@@ -806,26 +818,33 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
 // a stream that belongs to another device than the current one, or a full table with nothing to evict.
 //
 // Every device keeps a table of up to kFlatSlots stream handles; a stream's slot is its group of eight counters.
-// Behind every launch that uses a slot the library records an event of its own on the caller's stream
-// (flat_launch_recorded).  When the table is full, the least recently used slot whose event has completed — so no
-// launch that draws from its counters can still be running, whether or not its stream still exists — is given to
-// the new stream; handles of streams that may have been destroyed are never passed to the runtime.  A process that
-// creates and destroys streams therefore keeps the resident kernel for good.
+// Launches that use a slot are numbered, and the last workgroup of a launch writes that number into the slot's word
+// of a small pinned host array (flat_leave).  When the table is full, the least recently used slot whose word shows
+// its latest launch — so nothing can still be drawing from its counters, whether or not its stream still exists — is
+// given to the new stream.  The handles in the table are only ever compared, never passed to the runtime: a stream
+// may have been destroyed since.  A process that creates and destroys streams therefore keeps the resident kernel.
 struct FlatStreamStats { int64_t resident = 0, fallback = 0, evictions = 0; };
 static FlatStreamStats flat_stats[64];
 static std::mutex flat_mutex;
-struct FlatSlot { hipStream_t stream; uint64_t last_use; hipEvent_t done; bool recorded; };
-struct FlatDevice { uint32_t *base = nullptr; FlatSlot slots[kFlatSlots]; int used = 0; uint64_t clock = 0; };
+struct FlatSlot { hipStream_t stream; uint64_t last_use; uint32_t launches; };
+struct FlatDevice {
+    uint32_t *base = nullptr;
+    volatile uint32_t *done = nullptr;          // pinned host memory, one word per slot, written by the device
+    FlatSlot slots[kFlatSlots];
+    int used = 0;
+    uint64_t clock = 0;
+};
 static FlatDevice flat_devices[64];
+struct FlatLaunch { uint32_t *tickets; uint32_t *done_word; uint32_t number; };
 
-static uint32_t *flat_tickets_for(hipStream_t stream, int *dev_out, int *slot_out) {
+static bool flat_tickets_for(hipStream_t stream, FlatLaunch *launch) {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
-    auto fallback = [&]() -> uint32_t * {
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    auto fallback = [&]() -> bool {
         (void)hipGetLastError();
         std::lock_guard<std::mutex> lock(flat_mutex);
         flat_stats[dev].fallback++;
-        return nullptr;
+        return false;
     };
     if (stream == hipStreamPerThread) return fallback();
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
@@ -834,58 +853,47 @@ static uint32_t *flat_tickets_for(hipStream_t stream, int *dev_out, int *slot_ou
     if (hipStreamGetDevice(stream, &owner) != hipSuccess || (int)owner != dev) return fallback();   // counters are per device
     std::lock_guard<std::mutex> lock(flat_mutex);
     FlatDevice &d = flat_devices[dev];
-    if (d.base == nullptr && hipGetSymbolAddress((void **)&d.base, HIP_SYMBOL(flat_tickets)) != hipSuccess) {
-        (void)hipGetLastError();
-        d.base = nullptr;
-        flat_stats[dev].fallback++;
-        return nullptr;
+    if (d.base == nullptr) {
+        uint32_t *base = nullptr;
+        void *done = nullptr;
+        if (hipGetSymbolAddress((void **)&base, HIP_SYMBOL(flat_tickets)) != hipSuccess ||
+            hipHostMalloc(&done, kFlatSlots * sizeof(uint32_t), hipHostMallocDefault) != hipSuccess) {
+            (void)hipGetLastError();
+            flat_stats[dev].fallback++;
+            return false;
+        }
+        for (int k = 0; k < kFlatSlots; k++) ((uint32_t *)done)[k] = 0u;
+        d.base = base;
+        d.done = (volatile uint32_t *)done;
     }
     int slot = 0;
     while (slot < d.used && d.slots[slot].stream != stream) slot++;
     if (slot == d.used) {
         if (d.used < kFlatSlots) {
-            hipEvent_t ev = nullptr;
-            if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
-                (void)hipGetLastError();
-                flat_stats[dev].fallback++;
-                return nullptr;
-            }
-            d.slots[slot] = FlatSlot{stream, 0, ev, false};
+            d.slots[slot] = FlatSlot{stream, 0, 0u};
             d.used++;
         } else {
-            // least recently used first; a few event queries at most
             slot = -1;
             uint64_t tried_up_to = 0;
-            for (int attempt = 0; attempt < 8 && slot < 0; attempt++) {
+            for (int attempt = 0; attempt < 16 && slot < 0; attempt++) {       // least recently used first
                 int oldest = -1;
                 for (int k = 0; k < kFlatSlots; k++)
                     if (d.slots[k].last_use > tried_up_to && (oldest < 0 || d.slots[k].last_use < d.slots[oldest].last_use)) oldest = k;
                 if (oldest < 0) break;
                 tried_up_to = d.slots[oldest].last_use;
-                if (!d.slots[oldest].recorded) continue;                 // a launch whose end nothing marks: never handed on
-                if (hipEventQuery(d.slots[oldest].done) == hipSuccess) slot = oldest;
-                else (void)hipGetLastError();
+                if (d.done[oldest] == d.slots[oldest].launches) slot = oldest;
             }
-            if (slot < 0) { flat_stats[dev].fallback++; return nullptr; }
+            if (slot < 0) { flat_stats[dev].fallback++; return false; }
             flat_stats[dev].evictions++;
             d.slots[slot].stream = stream;
         }
     }
     d.slots[slot].last_use = ++d.clock;
-    d.slots[slot].recorded = false;             // until flat_launch_recorded has marked the end of the launch to come
+    launch->number = ++d.slots[slot].launches;
+    launch->tickets = d.base + slot * 4;
+    launch->done_word = (uint32_t *)d.done + slot;
     flat_stats[dev].resident++;
-    *dev_out = dev;
-    *slot_out = slot;
-    return d.base + slot * 4;
-}
-
-// Marks the end of the launch that was just issued with the counters of `slot` (see flat_tickets_for).
-static void flat_launch_recorded(int dev, int slot, hipStream_t stream) {
-    std::lock_guard<std::mutex> lock(flat_mutex);
-    FlatSlot &sl = flat_devices[dev].slots[slot];
-    if (sl.stream != stream) return;                                     // handed on in between: cannot happen while `recorded` is false
-    if (hipEventRecord(sl.done, stream) == hipSuccess) sl.recorded = true;
-    else (void)hipGetLastError();
+    return true;
 }
 
 template <typename T, int OP>
@@ -904,17 +912,17 @@ static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void 
         if (tiles < 1) tiles = 1;
         if (tiles > 0x7FFFFFFF) return fail(-1, "cross_entropy launcher: tensor too large for one launch");
         if (n % 8 == 0 && head == 0 && n >= kFlatStreamMinRow && total_vec >= kFlatStreamMinVec && total_vec < ((int64_t)1 << 32)) {
-            int dev = 0, slot = 0;
-            if (uint32_t *tickets = flat_tickets_for(s, &dev, &slot)) {
+            FlatLaunch fl;
+            if (flat_tickets_for(s, &fl)) {
+                uint32_t *tickets = fl.tickets;
                 const int cus = device_cu_count();
                 const unsigned grid = (unsigned)(cus >= 64 ? cus / 64 * 64 : 64);      // 8 XCDs x 8 counters
                 const int64_t per_tile = (int64_t)kFlatStreamThreads * kFlatStreamVecs;
                 hipLaunchKernelGGL(ce_flat_reset_kernel, dim3(1), dim3(64), 0, s, tickets, 2 * (grid / kFlatCounters));
                 hipLaunchKernelGGL((ce_flat_stream_kernel<T, OP>), dim3(grid), dim3(kFlatStreamThreads), 0, s, n, total_vec,
                                    (total_vec + per_tile - 1) / per_tile, (u32x4 *)x, (const float *)row_a, (const float *)row_b,
-                                   (const int32_t *)target, tickets);
+                                   (const int32_t *)target, tickets, fl.done_word, fl.number);
                 hipError_t e = hipGetLastError();
-                flat_launch_recorded(dev, slot, s);
                 return e == hipSuccess ? 0 : fail((int)e, who, e);
             }
         }

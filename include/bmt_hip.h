@@ -21,17 +21,18 @@
  *
  * State the library does keep (everything else is stateless, as the reference's launchers are):
  *   - host side: the parked worker threads of adam_cpu_*_launcher; per device, a table of up to 256
- *     stream handles (which stream uses which group of ticket counters below) with one event each, behind one mutex, the
+ *     stream handles (which stream uses which group of ticket counters below) behind one mutex, 1 KiB of pinned host memory, the
  *     looked-up addresses of the two device arrays, and the cached compute-unit count;
  *   - device side, two fixed arrays in the library's own code object, one copy per GPU: 32 KiB of
  *     ticket counters for the in-place cross-entropy kernels (eight counters per stream in the table)
  *     and the 4 MiB of partial sums of grad_stats_noalloc_launcher;
  *   - in a caller's buffer, only for the duration of a launch: long Adam launches keep four tile
  *     counters in the 16-bit parameter output (see adam_fp16_launcher).
- * The library records one event of its own on the caller's stream behind every launch that uses a table
- * entry.  When the table is full, the least recently used entry whose event has completed is given to the
- * new stream; if the entries looked at are all busy the launch runs the kernel that needs no counters
- * (same results, a few per cent slower).  Launches on a stream under
+ * Launches that use a table entry are numbered, and the last workgroup of each writes its number into a
+ * word of pinned host memory (1 KiB per device, allocated at the first such launch).  When the table is
+ * full, the least recently used entry whose latest launch has left is given to the new stream; if the
+ * entries looked at are all busy the launch runs the kernel that needs no counters (same results, a few
+ * per cent slower).  Stream handles in the table are only compared, never handed to the runtime.  Launches on a stream under
  * graph capture, on hipStreamPerThread or on a stream of another device always take that kernel.
  */
 #ifndef BMT_HIP_H

@@ -73,6 +73,10 @@ _ce_fwd = {
     "fp16": _sig("oracle_ce_forward_fp16", _i64, _i64, _p, _p, _p, _p, _i32),
     "bf16": _sig("oracle_ce_forward_bf16", _i64, _i64, _p, _p, _p, _p, _i32),
 }
+_ce_fwd_alt = {
+    "fp16": _sig("oracle_ce_forward_alt_fp16", _i64, _i64, _p, _p, _p, _p, _i32, _i32, _i32),
+    "bf16": _sig("oracle_ce_forward_alt_bf16", _i64, _i64, _p, _p, _p, _p, _i32, _i32, _i32),
+}
 _ce_bwd = {
     "fp16": _sig("oracle_ce_backward_fp16", _i64, _i64, _p, _p, _p, _i32),
     "bf16": _sig("oracle_ce_backward_bf16", _i64, _i64, _p, _p, _p, _i32),
@@ -159,6 +163,31 @@ def ce_forward(x_bits, target, ignore_index, dtype):
     softmax = np.empty((m, n), u16)
     out = np.empty(m, f32)
     _ce_fwd[dtype](m, n, _ptr(x_bits, u16), _ptr(target, i32), _ptr(softmax, u16), _ptr(out, f32), ignore_index)
+    return softmax, out
+
+
+EXP_LIBM, EXP_DOUBLE, EXP_WITHIN_ONE_ULP, EXP_WITHIN_TWO_ULP = 0, 1, 2, 3
+SUM_WARP32, SUM_WAVE64, SUM_DOUBLE = 0, 1, 2
+
+
+_alt_exp = _sig("oracle_alt_exp", _i64, _p, _p, _i32)
+
+
+def alt_exp(t: np.ndarray, exp_kind: int) -> np.ndarray:
+    """The exponential ce_forward_alt uses for `exp_kind`, element by element (float32 in, float32 out)."""
+    out = np.empty(t.size, f32)
+    _alt_exp(t.size, _ptr(t, f32), _ptr(out, f32), exp_kind)
+    return out
+
+
+def ce_forward_alt(x_bits, target, ignore_index, dtype, exp_kind=EXP_LIBM, sum_kind=SUM_WARP32):
+    """The forward expression evaluated another equally faithful way (which expf, which block-sum order); with the
+    defaults it is ce_forward.  Returns (softmax_bits[m,n], loss[m])."""
+    m, n = x_bits.shape
+    softmax = np.empty((m, n), u16)
+    out = np.empty(m, f32)
+    _ce_fwd_alt[dtype](m, n, _ptr(x_bits, u16), _ptr(target, i32), _ptr(softmax, u16), _ptr(out, f32), ignore_index,
+                       exp_kind, sum_kind)
     return softmax, out
 
 

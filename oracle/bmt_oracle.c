@@ -376,6 +376,91 @@ void oracle_ce_forward_bf16(int64_t m, int64_t n, const uint16_t *x, const int32
     ce_forward(m, n, x, target, softmax, out, ignore_index, bf16_to_float, float_to_bf16_rne);
 }
 
+/* The forward expression of cross_entropy.cu:17-42 evaluated in other ways that are equally faithful to the
+ * source: nothing in it fixes which expf the compiler links or how many lanes a warp has.
+ *   exp_kind 0: this host's libm expf (what ce_forward above uses);
+ *            1: exp in double precision, rounded to float (the correctly rounded value but for double rounding);
+ *            2: that value moved by one float ulp down, not at all, not at all or up, chosen by a fixed hash of
+ *               the argument's bits: a stand-in for any expf that is accurate to 1 ulp.  The reference's own expf
+ *               is the CUDA library's, whose documented maximum error is 2 ulp, so an evaluation that is 1 ulp
+ *               away from this host's libm on some arguments is as faithful to the source as libm's;
+ *            3: the same with steps of -2, -1, 0, 0, 0, 0, +1, +2 ulps: the full width that documented bound allows.
+ *   sum_kind 0: reduce.cuh's order on 32-lane warps (ce_forward above);
+ *            1: the same source on 64-lane wavefronts: 1024 strided partials, each wave folds with offsets
+ *               32..1, the 16 wave results fold with offsets 8..1;
+ *            2: the sum in double precision, rounded once.
+ * Used by tests to measure how far two faithful evaluations of the reference lie apart in 16-bit units. */
+static float alt_exp(float t, int exp_kind) {
+    if (exp_kind == 0) return expf(t);
+    float e = (float)exp((double)t);
+    if (exp_kind >= 2 && e > 0.f && isfinite(e)) {
+        uint32_t u, h;
+        memcpy(&u, &t, 4);
+        h = u * 2654435761u;
+        if (exp_kind == 2) {
+            h >>= 30;
+            if (h == 0) e = nextafterf(e, 0.f);
+            else if (h == 3) e = nextafterf(e, INFINITY);
+        } else {
+            h >>= 29;
+            if (h <= 1) e = nextafterf(e, 0.f);
+            if (h == 0) e = nextafterf(e, 0.f);
+            if (h >= 6) e = nextafterf(e, INFINITY);
+            if (h == 7) e = nextafterf(e, INFINITY);
+        }
+    }
+    return e;
+}
+void oracle_alt_exp(int64_t n, const float *t, float *out, int32_t exp_kind) {
+    for (int64_t i = 0; i < n; i++) out[i] = alt_exp(t[i], exp_kind);
+}
+static float block_sum_wave64(float *partial /* 1024, clobbered */) {
+    float wave[16];
+    for (int w = 0; w < 16; w++) {
+        float *x = partial + 64 * w;
+        for (int off = 32; off > 0; off >>= 1)
+            for (int l = 0; l < off; l++) x[l] += x[l + off];
+        wave[w] = x[0];
+    }
+    for (int off = 8; off > 0; off >>= 1)
+        for (int l = 0; l < off; l++) wave[l] += wave[l + off];
+    return wave[0];
+}
+static void ce_forward_alt(int64_t m, int64_t n, const uint16_t *x, const int32_t *target, uint16_t *softmax,
+                           float *out, int32_t ignore_index, cvt_in_fn in, cvt_out_fn outc, int exp_kind, int sum_kind) {
+    float partial[1024];
+    for (int64_t r = 0; r < m; r++) {
+        const uint16_t *row = x + r * n;
+        float mx = -INFINITY;
+        for (int64_t i = 0; i < n; i++) mx = fmaxf(in(row[i]), mx);
+        mx = fmaxf(mx, -1e6f);
+        float sum;
+        if (sum_kind == 2) {
+            double acc = 0.0;
+            for (int64_t i = 0; i < n; i++) acc += (double)alt_exp(in(row[i]) - mx, exp_kind);
+            sum = (float)acc;
+        } else {
+            for (int t = 0; t < 1024; t++) {
+                float s = 0.f;
+                for (int64_t i = t; i < n; i += 1024) s += alt_exp(in(row[i]) - mx, exp_kind);
+                partial[t] = s;
+            }
+            sum = sum_kind == 1 ? block_sum_wave64(partial) : ref_block_sum_1024(partial);
+        }
+        float S = (float)((double)sum + 1e-10);
+        for (int64_t i = 0; i < n; i++) softmax[r * n + i] = outc(alt_exp(in(row[i]) - mx, exp_kind) / S);
+        out[r] = target[r] != ignore_index ? (-in(row[target[r]]) + mx) + logf(S) : 0.f;
+    }
+}
+void oracle_ce_forward_alt_fp16(int64_t m, int64_t n, const uint16_t *x, const int32_t *target, uint16_t *softmax,
+                                float *out, int32_t ignore_index, int32_t exp_kind, int32_t sum_kind) {
+    ce_forward_alt(m, n, x, target, softmax, out, ignore_index, half_to_float, float_to_half_rne, exp_kind, sum_kind);
+}
+void oracle_ce_forward_alt_bf16(int64_t m, int64_t n, const uint16_t *x, const int32_t *target, uint16_t *softmax,
+                                float *out, int32_t ignore_index, int32_t exp_kind, int32_t sum_kind) {
+    ce_forward_alt(m, n, x, target, softmax, out, ignore_index, bf16_to_float, float_to_bf16_rne, exp_kind, sum_kind);
+}
+
 /* cross_entropy.cu:46-60 (fp16) / :104-121 (bf16): in place on the stored softmax,
  *   x_i = to16( i == t_r ? (x_i - 1) * v : x_i * v ),  v = grad_output[r].
  * ignore_index is not read: an ignored row (t_r = -100) simply never matches i. */

@@ -341,28 +341,41 @@ def test_around_the_launch_size_where_the_resident_grid_takes_over(flavour, n, o
     assert np.array_equal(bits16(hg), ho)
 
 
-def test_more_than_2_to_the_31_elements():
-    """Element counts beyond int32 (the reference's launcher takes `int n`): the last stretch of a
-    2^31 + 12345 element buffer must be stepped, and stepped correctly."""
+@pytest.mark.parametrize("flavour", ["bf16", "fp16"])
+def test_more_than_2_to_the_31_elements(flavour):
+    """Element counts beyond int32 (the reference's launchers take `int n`, adam_cuda.cu:76,103): the last stretch of a
+    2^31 + 12345 element buffer must be stepped, and stepped correctly, in both flavours."""
     n = (1 << 31) + 12345
+    fp16 = flavour == "fp16"
+    dt16 = torch.float16 if fp16 else torch.bfloat16
+    scale = 8.0 if fp16 else 1.0
     gen = torch.Generator(device="cuda").manual_seed(31)
-    before = {"p": torch.empty(n, device="cuda"), "m": torch.zeros(n, device="cuda"), "v": torch.zeros(n, device="cuda"),
-              "g": torch.empty(n, dtype=torch.bfloat16, device="cuda")}
-    _fill_(before["p"], 0.02, gen); _fill_(before["g"], 1e-3, gen)
+    before = {"p": torch.empty(n, device="cuda"), "m": torch.zeros(n, dtype=torch.float16 if fp16 else torch.float32, device="cuda"),
+              "v": torch.zeros(n, device="cuda"), "g": torch.empty(n, dtype=dt16, device="cuda")}
+    _fill_(before["p"], 0.02, gen); _fill_(before["g"], 1e-3 * scale, gen)
     slices = [(0, 4096), ((1 << 31) - 2048, (1 << 31) + 2048), (n - 12345, n)]
     snap = {k: {s: before[k][s[0]:s[1]].clone() for s in slices} for k in ("p", "m", "v", "g")}
-    h = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
-    F.adam_bf16(before["p"], h, before["g"], before["m"], before["v"], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 1)
+    h = torch.zeros(n, dtype=dt16, device="cuda")
+    fn = F.adam_fp16 if fp16 else F.adam_bf16
+    fn(before["p"], h, before["g"], before["m"], before["v"], 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, 1)
     bc1, bc2 = oracle.bias_corrections(0.9, 0.999, 1)
     for s in slices:
-        po, mo, vo = (snap[k][s].cpu().numpy().copy() for k in ("p", "m", "v"))
+        po, vo = (snap[k][s].cpu().numpy().copy() for k in ("p", "v"))
         ho = np.zeros(s[1] - s[0], np.uint16)
-        oracle.adam_gpu_bf16(po, ho, bits16(snap["g"][s]), mo, vo, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, bc1, bc2)
+        if fp16:
+            mo = bits16(snap["m"][s])
+            oracle.adam_gpu_fp16(po, ho, bits16(snap["g"][s]), mo, vo, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, bc1, bc2)
+            assert np.array_equal(bits16(before["m"][s[0]:s[1]]), mo), s
+        else:
+            mo = snap["m"][s].cpu().numpy().copy()
+            oracle.adam_gpu_bf16(po, ho, bits16(snap["g"][s]), mo, vo, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, bc1, bc2)
+            assert np.array_equal(f32_bits(before["m"][s[0]:s[1]].cpu().numpy()), f32_bits(mo)), s
         assert np.array_equal(f32_bits(before["p"][s[0]:s[1]].cpu().numpy()), f32_bits(po)), s
         assert np.array_equal(f32_bits(before["v"][s[0]:s[1]].cpu().numpy()), f32_bits(vo)), s
         assert np.array_equal(bits16(h[s[0]:s[1]]), ho), s
-    assert torch.count_nonzero(before["v"][-(1 << 20):]) == (1 << 20)
-    del before, h
+    # every element of the last stretch was stepped (a gradient that rounded to zero leaves v at zero)
+    assert torch.count_nonzero(before["v"][-(1 << 20):]) == torch.count_nonzero(before["g"][-(1 << 20):]) > (1 << 20) - 64
+    del before, h, snap
     torch.cuda.empty_cache()
 
 
@@ -443,22 +456,28 @@ def _checksum(t, chunk=1 << 28):
     return total & ((1 << 64) - 1)
 
 
-def test_whole_model_flat_buffer_equals_tensor_list():
-    """6,738,415,616 elements (a 7B-parameter model's state, 108 GB): one launch over the flat buffers.
-    Seeded slices — the first and last elements, and a stretch across element 2^32 — are checked against
-    the oracle bit for bit; then the identical inputs are stepped tensor by tensor (291 tensors of the
+@pytest.mark.parametrize("flavour", ["bf16", "fp16"])
+def test_whole_model_flat_buffer_equals_tensor_list(flavour):
+    """6,738,415,616 elements (a 7B-parameter model's state, 108 GB; 94 GB in the fp16 flavour): one launch over the
+    flat buffers.  Seeded slices — the first and last elements, and a stretch across element 2^32 — are checked
+    against the oracle bit for bit; then the identical inputs are stepped tensor by tensor (291 tensors of the
     Llama-7B shapes, one launch each) and every output buffer must have the same checksum."""
+    fp16 = flavour == "fp16"
+    dt16 = torch.float16 if fp16 else torch.bfloat16
+    scale = 64.0 if fp16 else 1.0
+    fn = F.adam_fp16 if fp16 else F.adam_bf16
     layer = [4096 * 4096] * 4 + [4096 * 11008] * 3 + [4096] * 2
     shapes = [32000 * 4096] + layer * 32 + [4096, 32000 * 4096]
     n = sum(shapes)
     assert n == 6_738_415_616 and len(shapes) == 291
-    bufs = {"h": torch.empty(n, dtype=torch.bfloat16, device="cuda"), "g": torch.empty(n, dtype=torch.bfloat16, device="cuda"),
-            "p": torch.empty(n, device="cuda"), "m": torch.empty(n, device="cuda"), "v": torch.empty(n, device="cuda")}
+    bufs = {"h": torch.empty(n, dtype=dt16, device="cuda"), "g": torch.empty(n, dtype=dt16, device="cuda"),
+            "p": torch.empty(n, device="cuda"), "m": torch.empty(n, dtype=torch.float16 if fp16 else torch.float32, device="cuda"),
+            "v": torch.empty(n, device="cuda")}
 
     def fill():
         gen = torch.Generator(device="cuda").manual_seed(4)
-        _fill_(bufs["p"], 0.02, gen); _fill_(bufs["m"], 1e-4, gen); _fill_(bufs["v"], 1e-6, gen, absolute=True)
-        _fill_(bufs["g"], 1e-3, gen)
+        _fill_(bufs["p"], 0.02, gen); _fill_(bufs["m"], 1e-4 * scale, gen); _fill_(bufs["v"], 1e-6 * scale, gen, absolute=True)
+        _fill_(bufs["g"], 1e-3 * scale, gen)
         bufs["h"].zero_()
 
     fill()
@@ -466,14 +485,20 @@ def test_whole_model_flat_buffer_equals_tensor_list():
     starts = [0, n - 70000, (1 << 32) - 30000] + [int(s) for s in rnd.integers(0, n - 70000, 5)]
     slices = [(s, s + 65536 + 7) for s in starts]
     snap = {k: {s: bufs[k][s[0]:s[1]].clone() for s in slices} for k in ("p", "m", "v", "g")}
-    F.adam_bf16(bufs["p"], bufs["h"], bufs["g"], bufs["m"], bufs["v"], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100)
+    fn(bufs["p"], bufs["h"], bufs["g"], bufs["m"], bufs["v"], 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, 100)
     bc1, bc2 = oracle.bias_corrections(0.9, 0.999, 100)
     for s in slices:
-        po, mo, vo = (snap[k][s].cpu().numpy().copy() for k in ("p", "m", "v"))
+        po, vo = (snap[k][s].cpu().numpy().copy() for k in ("p", "v"))
         ho = np.zeros(s[1] - s[0], np.uint16)
-        oracle.adam_gpu_bf16(po, ho, bits16(snap["g"][s]), mo, vo, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, bc1, bc2)
+        if fp16:
+            mo = bits16(snap["m"][s])
+            oracle.adam_gpu_fp16(po, ho, bits16(snap["g"][s]), mo, vo, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, bc1, bc2)
+            assert np.array_equal(bits16(bufs["m"][s[0]:s[1]]), mo), s
+        else:
+            mo = snap["m"][s].cpu().numpy().copy()
+            oracle.adam_gpu_bf16(po, ho, bits16(snap["g"][s]), mo, vo, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, bc1, bc2)
+            assert np.array_equal(f32_bits(bufs["m"][s[0]:s[1]].cpu().numpy()), f32_bits(mo)), s
         assert np.array_equal(f32_bits(bufs["p"][s[0]:s[1]].cpu().numpy()), f32_bits(po)), s
-        assert np.array_equal(f32_bits(bufs["m"][s[0]:s[1]].cpu().numpy()), f32_bits(mo)), s
         assert np.array_equal(f32_bits(bufs["v"][s[0]:s[1]].cpu().numpy()), f32_bits(vo)), s
         assert np.array_equal(bits16(bufs["h"][s[0]:s[1]]), ho), s
     flat = {k: _checksum(bufs[k]) for k in ("p", "m", "v", "h")}
@@ -482,9 +507,10 @@ def test_whole_model_flat_buffer_equals_tensor_list():
     lo = 0
     for size in shapes:
         hi = lo + size
-        F.adam_bf16(bufs["p"][lo:hi], bufs["h"][lo:hi], bufs["g"][lo:hi], bufs["m"][lo:hi], bufs["v"][lo:hi],
-                    0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100)
+        fn(bufs["p"][lo:hi], bufs["h"][lo:hi], bufs["g"][lo:hi], bufs["m"][lo:hi], bufs["v"][lo:hi],
+           0.9, 0.999, 1e-8, 1e-3, scale, 0.01, 100)
         lo = hi
     assert {k: _checksum(bufs[k]) for k in ("p", "m", "v", "h")} == flat
+    del snap
     bufs.clear()
     torch.cuda.empty_cache()

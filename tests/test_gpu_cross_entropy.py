@@ -44,14 +44,24 @@ WIDTHS = [1, 2, 3, 7, 8, 9, 10, 15, 16, 17, 90, 100, 512, 513, 520, 1000, 1001, 
 @pytest.mark.parametrize("name,dtype", DTYPES)
 @pytest.mark.parametrize("n", WIDTHS)
 def test_forward_against_oracle(name, dtype, n):
-    m = 37 if n <= 4096 else 5
+    m = max(5, min(2000, 1_000_000 // n))          # about a million elements per case
     x, t = _case(m, n, dtype, seed=n)
     softmax, loss = _forward_gpu(x, t)
     want_soft, want_loss = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
     assert ulp_distance16(bits16(softmax), want_soft).max() <= 1
     # rarely off by its one ulp: more often for fp16 values in the normal range, whose ulp is 2^-11 of the value,
-    # than for bf16 (2^-8) or the subnormal fp16 values of long rows; the benchmark shapes have a test of their own
-    assert (bits16(softmax) != want_soft).sum() <= 3 + (1e-3 if name == "fp16" else 2e-4) * m * n
+    # than for bf16 (2^-8) or the subnormal fp16 values of long rows.  Measured over 3 M elements per width: fp16
+    # 1.6e-4 to 2.5e-4 up to 512 classes, 1e-4 at 4,096, 4e-5 at 32,000, 1e-5 beyond 100,000; bf16 1e-5 to 6e-5 at
+    # every width; two-class rows 5e-4 in both types.  The bounds leave a factor of 1.5 to 2 for the sample of about a
+    # million elements (the differing elements of a row move together with its sum); the benchmark shapes have a test
+    # of their own.
+    if n <= 2:
+        allowed = 1e-3
+    elif name == "fp16":
+        allowed = 4e-4 if n <= 8192 else 1.5e-4
+    else:
+        allowed = 1.5e-4          # a single row can reach 2e-4 when its sum lands close to a rounding boundary of many quotients
+    assert (bits16(softmax) != want_soft).sum() <= 3 + allowed * m * n
     np.testing.assert_allclose(loss.cpu().numpy(), want_loss, rtol=2e-6, atol=2e-6)
     ref32 = torch.nn.functional.cross_entropy(x.float(), t.long(), ignore_index=-100, reduction="none").numpy()
     np.testing.assert_allclose(loss.cpu().numpy(), ref32, rtol=1e-3, atol=1e-6)

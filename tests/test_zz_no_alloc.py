@@ -61,3 +61,46 @@ def test_nothing_is_allocated_and_too_large_is_refused():
     with pytest.raises(RuntimeError, match="2\\^36"):
         C.grad_stats_noalloc_launcher((1 << 36) + (1 << 20), g.data_ptr(), 1, sumsq.data_ptr(), flag.data_ptr(), stream)
     C.grad_stats_noalloc_launcher(0, 0, 1, 0, 0, stream)       # n <= 0: no-op
+
+
+def test_captured_in_a_graph_and_replayed():
+    """The call is meant for code under graph capture.  Captured on a side stream (after one eager call on the same
+    device, so that the array's address has been looked up outside the capture), then replayed five times on that
+    stream with new gradient contents and eager work in between: every replay gives the bits of the workspace form,
+    and no device memory is taken by capture or replay."""
+    n = (1 << 22) + 777
+    g = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+    sumsq = torch.zeros(1, dtype=torch.float64, device="cuda")
+    flag = torch.zeros(1, dtype=torch.uint8, device="cuda")
+    work = torch.empty(C.grad_stats_workspace_floats(n), dtype=torch.float32, device="cuda")
+    want_sumsq = torch.zeros(1, dtype=torch.float64, device="cuda")
+    want_flag = torch.zeros(1, dtype=torch.uint8, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        C.grad_stats_noalloc_launcher(n, g.data_ptr(), 1, sumsq.data_ptr(), flag.data_ptr(), side.cuda_stream)   # warm-up
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            sumsq.zero_()                                   # a fill kernel, not a memset node
+            flag.zero_()
+            C.grad_stats_noalloc_launcher(n, g.data_ptr(), 1, sumsq.data_ptr(), flag.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    gen = torch.Generator(device="cuda").manual_seed(8)
+    for replay in range(5):
+        g.copy_((torch.randn(n, generator=gen, device="cuda") * (replay + 1)).bfloat16())     # eager work between replays
+        if replay == 3:
+            g[n - 5] = float("nan")
+        want_sumsq.zero_(); want_flag.zero_()
+        C.grad_stats_bf16_launcher(n, g.data_ptr(), want_sumsq.data_ptr(), want_flag.data_ptr(), work.data_ptr(),
+                                   torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(flag.item()) == int(want_flag.item()) == (1 if replay == 3 else 0), replay
+        if replay != 3:
+            assert sumsq.view(torch.int64).item() == want_sumsq.view(torch.int64).item(), replay
+    del gen
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] >= free_before - (64 << 20)      # torch's generator may cache a block; no growth per replay
