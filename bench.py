@@ -148,6 +148,34 @@ def cpu_baseline():
                                         "20 steps back to back, same buffers and cores as the reference's kernel above")
     except Exception as exc:                      # the baseline must not sink the GPU numbers
         out["product_host_adam"] = {"error": repr(exc)}
+    # The same kernels on a working set no cache holds (N = 2^27: 1.9 GB of state and gradients, 3.76 GB moved per
+    # step).  At N = 2^24 the 235 MB working set fits the last-level caches of large hosts, and the figures above then
+    # say more about the cache than about the kernel: they have read 350 to 1,400 GB/s for the same code on
+    # different boxes of this pool.
+    try:
+        nb = 1 << 27
+        pb = np.full(nb, 0.01, np.float32); mb = np.zeros(nb, np.float32); vb = np.zeros(nb, np.float32)
+        hb = np.zeros(nb, np.uint16)
+        gbig = np.tile(grads[0], nb // n)
+        big = {}
+        from bmtrain_amd import C as _C
+        runs = [("product_fp16", _C.adam_cpu_fp16_launcher, 1024.0)]
+        if ref is not None:
+            runs.insert(0, ("reference_fp16", ref.adam_cpu_fp16_launcher, 1024.0))
+        for label, launcher, scale in runs:
+            ts = []
+            for k in range(6):
+                bc1, bc2 = oracle.bias_corrections(0.9, 0.999, k + 1)
+                t0 = time.perf_counter()
+                launcher(nb, pb.ctypes.data, hb.ctypes.data, 0, gbig.ctypes.data, mb.ctypes.data, vb.ctypes.data,
+                         0.9, 0.999, 1e-8, 1e-3, scale, 0.01, bc1, bc2)
+                ts.append(time.perf_counter() - t0)
+            ts = sorted(ts[1:])
+            big[label] = {"GBps_median": round(ADAM_BF16_BYTES * nb / ts[len(ts) // 2] / 1e9, 1), "ms_median": round(ts[len(ts) // 2] * 1e3, 2)}
+        out["adam_cpu_N_2^27_beyond_cache"] = dict(big, cores=cores, sample="adam_cpu fp16 grads, N=2^27, 5 steps timed after one warm-up")
+        del pb, mb, vb, hb, gbig
+    except Exception as exc:
+        out["adam_cpu_N_2^27_beyond_cache"] = {"error": repr(exc)}
     # CPU cross-entropy (torch), fp32 as FusedCrossEntropy itself does for fp32 input
     torch.set_num_threads(cores)
     for key, rows, classes, std, every in (("ce", 256, 128256, 3.0, 20), ("ce_32000", 1024, 32000, 2.0, 10)):
@@ -211,15 +239,35 @@ def other_workloads(torch, dev, LF, OF, iters=20):
     out["adam_bf16_one_block_202M"] = entry(
         timed(lambda: OF.adam_bf16(p32, p16, grad, mom, var, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100)), ADAM_BF16_BYTES * n,
         buffers="five separate allocations made for this measurement")
-    h16, g16, m16 = p16.view(torch.float16), grad.view(torch.float16), mom.view(torch.float16)[:n]
-    g16.copy_(grad.float().mul_(1024.0)); m16.zero_(); fill_normal_(var, 1e-3, gen, absolute=True)
-    out["adam_fp16_one_block_202M"] = entry(
-        timed(lambda: OF.adam_fp16(p32, h16, g16, m16, var, 0.9, 0.999, 1e-8, 1e-3, 1024.0, 0.01, 100)), 24 * n,
-        bytes_per_element=24)
     sumsq = torch.zeros(1, dtype=torch.float64, device=dev)
     flag = torch.zeros(1, dtype=torch.uint8, device=dev)
     out["grad_stats_bf16_202M"] = entry(timed(lambda: OF.grad_stats(grad, sumsq, flag)), 2 * n)
-    del p16, grad, p32, mom, var, h16, g16, m16
+    # single mid-size tensors, as per-tensor stepping of a model meets them: below 12,582,912 elements a bf16 launch is
+    # one workgroup per tile, from there on the resident grid (launches back to back, so each figure holds one launch gap)
+    for label, k in (("adam_bf16_one_tensor_2^22", 1 << 22), ("adam_bf16_one_tensor_2^23", 1 << 23),
+                     ("adam_bf16_one_tensor_12.6M", 3 << 22), ("adam_bf16_one_tensor_4096x4096", 1 << 24),
+                     ("adam_bf16_one_tensor_11008x4096", 11008 * 4096)):
+        out[label] = entry(timed_batches(torch, lambda: OF.adam_bf16(p32[:k], p16[:k], grad[:k], mom[:k], var[:k], 0.9, 0.999, 1e-8, 1e-3,
+                                                                     1.0, 0.01, 100), 64, per_batch=16), ADAM_BF16_BYTES * k, elements=k)
+    del p16, grad, p32, mom, var
+    torch.cuda.empty_cache()
+    # the fp16 flavour (24 B / element: the first moment is a 16-bit array, kept multiplied by the loss scale), on buffers of its own
+    p32, var = torch.empty(n, device=dev), torch.empty(n, device=dev)
+    h16, g16, m16 = (torch.empty(n, dtype=torch.float16, device=dev) for _ in range(3))
+    fill_normal_(p32, 0.02, gen); fill_normal_(var, 1e-3, gen, absolute=True); fill_normal_(g16, 1.0, gen); m16.zero_()
+    out["adam_fp16_one_block_202M"] = entry(
+        timed(lambda: OF.adam_fp16(p32, h16, g16, m16, var, 0.9, 0.999, 1e-8, 1e-3, 1024.0, 0.01, 100)), 24 * n,
+        bytes_per_element=24)
+    del p32, var, h16, g16, m16
+    torch.cuda.empty_cache()
+    nf = LLAMA7B_ELEMENTS
+    p32, var = torch.empty(nf, device=dev), torch.empty(nf, device=dev)
+    h16, g16, m16 = (torch.empty(nf, dtype=torch.float16, device=dev) for _ in range(3))
+    fill_normal_(p32, 0.02, gen); fill_normal_(var, 1e-3, gen, absolute=True); fill_normal_(g16, 1.0, gen); m16.zero_()
+    out["adam_fp16_6.74B"] = entry(
+        timed_batches(torch, lambda: OF.adam_fp16(p32, h16, g16, m16, var, 0.9, 0.999, 1e-8, 1e-3, 1024.0, 0.01, 100), 6, per_batch=1),
+        24 * nf, bytes_per_element=24, elements=nf)
+    del p32, var, h16, g16, m16
     torch.cuda.empty_cache()
 
     n16 = 1 << 30
@@ -470,6 +518,31 @@ def main():
     assert flag.item() == 0, "synthetic gradients are finite"
     assert torch.isfinite(row_loss).all()
 
+    # The cross-entropy kernels once more, outside the step: the forward launched four times per event pair (one pair
+    # around a single sub-millisecond launch also holds the gap to the launch before it), and the backward "cold":
+    # between forward and backward a scan over the 13.5 GB of gradients sweeps the caches, where the step's own
+    # backward starts right after the forward that wrote its input.
+    ce_side = None
+    if not args.small:
+        fwd = timed_batches(torch, lambda: LF.cross_entropy_forward(rows, classes, logits, target, softmax, row_loss, -100), 24)
+        cold = []
+        for _ in range(8):
+            LF.cross_entropy_forward(rows, classes, logits, target, softmax, row_loss, -100)
+            LF.has_inf_nan(grad, flag)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            LF.cross_entropy_backward_inplace(rows, classes, grad_output, target, softmax, -100)
+            b.record()
+            b.synchronize()
+            cold.append(a.elapsed_time(b))
+        cold.sort()
+        fb = (4 * classes + 8) * rows
+        ce_side = {"ce_forward_back_to_back": {"ms": round(fwd[0], 4), "ms_median": round(fwd[1], 4), "ms_min": round(fwd[2], 4),
+                                               "frac": round(fb / (fwd[0] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
+                   "ce_backward_cold": {"ms": round(sum(cold) / len(cold), 4), "ms_median": round(cold[len(cold) // 2], 4),
+                                        "ms_min": round(cold[0], 4),
+                                        "frac": round(fb / (sum(cold) / len(cold) * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}}
+
     if args.calibrate_copy:
         softmax.copy_(logits)
         torch.cuda.synchronize()
@@ -530,6 +603,8 @@ def main():
                            "frac": round(ce_gbps / HBM_PEAK_GBPS, 4), "bytes_per_row": ce_bytes_per_row(classes)},
         },
     }
+    if ce_side:
+        result["other_kernels"].update(ce_side)
     side = not (args.small or args.no_other_workloads)
     block_in_place = model_side = None
     if side:

@@ -331,14 +331,24 @@ __global__ __launch_bounds__(kSmallThreads) void ce_forward_small_kernel(
 // altogether runs no faster.
 // Fine-grained load/compute interleaving in both sweeps lets the 32 waves of a CU hide each
 // other's latencies, which a whole-row-resident scheme with one or two workgroups per CU cannot.
-template <typename T, int RK, int LK>
+//
+// XR > 0 (rows of more than 12,288 vectors) keeps three more chunks: one in what is left of the CU's LDS — two
+// workgroups share 160 KiB, so all lanes but the last 16 find room for a fifth vector — and the two after it in
+// registers (58 VGPRs), and issues the four loads of the register part before it folds the first of them.  Together
+// 0.8 % at 128,256 classes (0.7597 -> 0.7529 ms, nine alternating rounds in one process); on rows that have no
+// dropped part the same code is 2 % slower, hence the condition.  Chunks are folded into the running sums two at a
+// time in row order either way, so the results do not depend on RK / LK / XR.
+template <typename T, int RK, int LK, int XR>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void ce_forward_retain_kernel(
     int32_t n, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
     uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index, int32_t chunks) {
     constexpr int THREADS = 1024;
     constexpr int GROUP = 2;
     static_assert(RK % GROUP == 0 && LK % GROUP == 0, "chunk counts must be even");   // and so is `chunks`
-    extern __shared__ u32x4 staged[];  // LK * 1024 vectors
+    static_assert(XR == 0 || XR == 2, "none, or chunk RK + LK in LDS and the two after it in registers");
+    constexpr int kPartialLanes = THREADS - 16;                 // lanes whose vector of chunk RK + LK fits into LDS
+    constexpr int DROP0 = RK + LK + (XR > 0 ? 2 * GROUP : 0);   // first chunk that every lane fetches twice
+    extern __shared__ u32x4 staged[];  // LK * 1024 vectors, and kPartialLanes more when XR > 0
     __shared__ float slots[2][THREADS / kWave];
     const int64_t row = blockIdx.x;
     const RowSpan sp = row_span(x, row, n);
@@ -366,19 +376,37 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
         for (int g = 0; g < GROUP; g++) vec_sumexp<T>(v[g], m, s);
     };
     u32x4 w[RK > 0 ? RK : 1];
+    u32x4 wx = pad4, wy = pad4;
     // register part
+    if constexpr (XR > 0) {
 #pragma unroll
-    for (int c0 = 0; c0 < RK; c0 += GROUP) {
-        u32x4 v[GROUP];
-#pragma unroll
-        for (int g = 0; g < GROUP; g++) {
-            const int j = (c0 + g) * THREADS + tid;
-            v[g] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
+        for (int c = 0; c < RK; c++) {
+            const int j = c * THREADS + tid;
+            w[c] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
         }
-        absorb(v, c0);
-#pragma unroll
-        for (int g = 0; g < GROUP; g++) w[c0 + g] = v[g];
         __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c0 = 0; c0 < RK; c0 += GROUP) {
+            u32x4 v[GROUP];
+#pragma unroll
+            for (int g = 0; g < GROUP; g++) v[g] = w[c0 + g];
+            absorb(v, c0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+#pragma unroll
+        for (int c0 = 0; c0 < RK; c0 += GROUP) {
+            u32x4 v[GROUP];
+#pragma unroll
+            for (int g = 0; g < GROUP; g++) {
+                const int j = (c0 + g) * THREADS + tid;
+                v[g] = j < nvec ? __builtin_nontemporal_load(xr + j) : pad4;
+            }
+            absorb(v, c0);
+#pragma unroll
+            for (int g = 0; g < GROUP; g++) w[c0 + g] = v[g];
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
     // LDS part
 #pragma unroll 1
@@ -393,9 +421,31 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
 #pragma unroll
         for (int g = 0; g < GROUP; g++) staged[(c0 + g - RK) * THREADS + tid] = v[g];
     }
+    if constexpr (XR > 0) {
+        // chunk RK + LK: to LDS where there is room (the last 16 lanes fetch theirs twice), RK + LK + 1: register
+        {
+            u32x4 v[GROUP];
+            const int j0 = (RK + LK) * THREADS + tid, j1 = j0 + THREADS;
+            if (tid < kPartialLanes) v[0] = j0 < nvec ? __builtin_nontemporal_load(xr + j0) : pad4;
+            else v[0] = j0 < nvec ? xr[j0] : pad4;
+            v[1] = j1 < nvec ? __builtin_nontemporal_load(xr + j1) : pad4;
+            absorb(v, RK + LK);
+            if (tid < kPartialLanes) staged[LK * THREADS + tid] = v[0];
+            wx = v[1];
+        }
+        // chunk RK + LK + 2: register, RK + LK + 3: fetched twice
+        {
+            u32x4 v[GROUP];
+            const int j0 = (RK + LK + 2) * THREADS + tid, j1 = j0 + THREADS;
+            v[0] = j0 < nvec ? __builtin_nontemporal_load(xr + j0) : pad4;
+            v[1] = j1 < nvec ? xr[j1] : pad4;
+            absorb(v, RK + LK + 2);
+            wy = v[0];
+        }
+    }
     // dropped part: default cache policy, so that the second fetch finds it in L2 or the memory-side cache
 #pragma unroll 1
-    for (int c0 = RK + LK; c0 < chunks; c0 += GROUP) {
+    for (int c0 = DROP0; c0 < chunks; c0 += GROUP) {
         u32x4 v[GROUP];
 #pragma unroll
         for (int g = 0; g < GROUP; g++) {
@@ -422,7 +472,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
 
     // dropped part, last fetched first; its lines are not needed again (non-temporal)
 #pragma unroll 1
-    for (int c0 = chunks - GROUP; c0 >= RK + LK; c0 -= GROUP) {
+    for (int c0 = chunks - GROUP; c0 >= DROP0; c0 -= GROUP) {
         u32x4 v[GROUP];
 #pragma unroll
         for (int g = GROUP - 1; g >= 0; g--) {
@@ -435,6 +485,22 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
             if (j < nvec) __builtin_nontemporal_store(vec_softmax<T>(v[g], M, rs), sr + j);
         }
         __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (XR > 0) {
+        {
+            const int j0 = (RK + LK + 2) * THREADS + tid, j1 = j0 + THREADS;
+            const u32x4 v1 = j1 < nvec ? __builtin_nontemporal_load(xr + j1) : pad4;
+            if (j1 < nvec) __builtin_nontemporal_store(vec_softmax<T>(v1, M, rs), sr + j1);
+            if (j0 < nvec) __builtin_nontemporal_store(vec_softmax<T>(reread(wy), M, rs), sr + j0);
+        }
+        {
+            const int j0 = (RK + LK) * THREADS + tid, j1 = j0 + THREADS;
+            u32x4 v0 = pad4;
+            if (tid >= kPartialLanes && j0 < nvec) v0 = __builtin_nontemporal_load(xr + j0);
+            if (j1 < nvec) __builtin_nontemporal_store(vec_softmax<T>(reread(wx), M, rs), sr + j1);
+            if (tid < kPartialLanes) v0 = staged[LK * THREADS + tid];
+            if (j0 < nvec) __builtin_nontemporal_store(vec_softmax<T>(v0, M, rs), sr + j0);
+        }
     }
     // LDS part (each lane reads the slots it wrote itself)
 #pragma unroll 1
@@ -756,10 +822,10 @@ static int flat_grid(int64_t work_items, int threads_times_unroll) {
                            (uint16_t *)softmax, (float *)output, ignore_index);                                    \
     } while (0)
 
-#define BMT_CE_RETAIN(CHUNKS, RK, LK)                                                                              \
+#define BMT_CE_RETAIN(CHUNKS, RK, LK, XR)                                                                          \
     do {                                                                                                           \
-        auto kern = ce_forward_retain_kernel<T, RK, LK>;                                                           \
-        const size_t lds = (size_t)(LK) * 1024 * sizeof(u32x4);                                                    \
+        auto kern = ce_forward_retain_kernel<T, RK, LK, XR>;                                                       \
+        const size_t lds = ((size_t)(LK) * 1024 + ((XR) > 0 ? 1024 - 16 : 0)) * sizeof(u32x4);                     \
         static std::atomic<uint64_t> allowed{0};   /* devices on which this kernel may use `lds` bytes */         \
         int dev = 0;                                                                                               \
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 63;                                    \
@@ -801,9 +867,11 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
         else if (nvec <= 3072) BMT_CE_ROW(1024, 3);
         else if (nvec <= 4096) BMT_CE_ROW(1024, 4);
         // up to 65,536 elements: 4 vectors per lane in registers, the rest in LDS, two workgroups per CU
-        else if (nvec <= 6144) BMT_CE_RETAIN(6, 2, 4);
-        // longer rows: 8 vectors per lane kept, the rest fetched twice
-        else BMT_CE_RETAIN(2 * ((nvec + 2047) / 2048), 4, 4);
+        else if (nvec <= 6144) BMT_CE_RETAIN(6, 2, 4, 0);
+        // up to 98,304 elements: 8 vectors per lane kept, the rest fetched twice
+        else if (nvec <= 12288) BMT_CE_RETAIN(2 * ((nvec + 2047) / 2048), 4, 4, 0);
+        // longer rows: 11 vectors per lane kept (all but 16 lanes)
+        else BMT_CE_RETAIN(2 * ((nvec + 2047) / 2048), 4, 4, 2);
     } else {
         hipLaunchKernelGGL((ce_forward_sweep_kernel<T>), dim3((unsigned)m), dim3(kSweepThreads), 0, s, n,
                            (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,
