@@ -227,8 +227,12 @@ __global__ void adam_stream_reset_kernel(u32x2 *p16, int64_t nvec, uint32_t firs
 }
 // The grid of the resident kernels: one workgroup per compute unit, rounded down to a multiple of 32
 // (8 XCDs x 4 counters), at least 32.
-static unsigned stream_grid() {
-    const int cus = device_cu_count();
+// The fp16 flavour moves fewer bytes per tile (its first moment is a 16-bit array) and runs 1 % faster with a
+// quarter more workgroups (1.6 B elements: 81.3 % of peak with 320 workgroups, 80.1 % with 256, 80.6 % with 384, 78 % with
+// 512); the bf16 flavour is fastest with exactly one per compute unit (84 %; 288: 82 %, 320: 81 %).
+static unsigned stream_grid(bool fp16 = false) {
+    int cus = device_cu_count();
+    if (fp16) cus += cus / 4;
     return (unsigned)(cus >= 32 ? cus / 32 * 32 : 32);
 }
 // Workgroup b draws from counter (b / 8) % 4.  Its first two tickets need no atomic: it is workgroup number q
@@ -455,8 +459,8 @@ static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16
             u32x2 *out16 = (u32x2 *)(p16 + head);
             if (nvec >= kStreamMinVecFp16) {
                 const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
-                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec, stream_grid() / 2);
-                hipLaunchKernelGGL((adam_stream_kernel<true>), dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
+                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec, stream_grid(true) / 2);
+                hipLaunchKernelGGL((adam_stream_kernel<true>), dim3(stream_grid(true)), dim3(kStreamThreads), 0, s, nvec,
                                    ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
                                    (f32x4 *)(v + head), h);
                 hipLaunchKernelGGL((adam_stream_finish_kernel<Half>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
@@ -721,8 +725,8 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
         }
         if (counters_clear && groups >= (FP16 ? kStreamMinVecFp16 : kStreamMinVecBf16)) {
             hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, (u32x2 *)batch.p16[batch.counter_tensor], most,
-                               stream_grid() / 2);
-            hipLaunchKernelGGL((adam_stream_multi_kernel<FP16>), dim3(stream_grid()), dim3(kStreamThreads), 0, s,
+                               stream_grid(FP16) / 2);
+            hipLaunchKernelGGL((adam_stream_multi_kernel<FP16>), dim3(stream_grid(FP16)), dim3(kStreamThreads), 0, s,
                                batch, h);
             hipLaunchKernelGGL((adam_stream_multi_finish_kernel<FP16>), dim3(1), dim3(4 * kBatch + 64), 0, s, batch, h);
         } else {
