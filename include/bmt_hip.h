@@ -166,9 +166,11 @@ BMT_API int fused_softmax_inplace_bf16_launcher(int32_t m, int32_t n, void *logi
  * `count` tensors that share their hyper-parameters (same group, same step count) in as few launches as
  * possible; per element the arithmetic is that of adam_{fp16,bf16}_launcher, bit for bit.
  * `tensors` is a host array; `m` is float[n] for bf16 and half[n] for fp16.  Entries with n <= 0 are skipped.
- * param_16 is output only; a launch over 2^24 elements or more keeps four tile counters in the
- * param_16 of its largest tensor while it runs (as adam_fp16_launcher does), and returns -1 if a param_16
- * overlaps an input of the same tensor.
+ * param_16 is output only; a launch over 2^24 elements or more (bf16: 12,582,912 or more) keeps four tile counters in the
+ * param_16 of its largest tensor while it runs (as adam_fp16_launcher does).  The whole table is checked before
+ * the first launch: the call returns -1, and no tensor has been stepped, if any entry has a null pointer or a
+ * param_16 that overlaps an input of the same tensor.  A batch in which another entry shares memory with the
+ * counters' place runs on the kernel that keeps no counters.
  */
 typedef struct bmt_adam_tensor {
     void *param_fp32;
