@@ -61,3 +61,28 @@ def test_argument_count_is_checked_and_degenerate_sizes_are_noops():
     C.cross_entropy_backward_inplace_bf16_launcher(4, 0, 0, 0, 0, -100, 0)
     with pytest.raises(RuntimeError, match="null pointer"):
         C.adam_cpu_fp16_launcher(4, 0, 0, 0, 0, 0, 0, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.0, 0.1, 0.001)
+
+
+def test_header_is_plain_c_and_the_documented_bindings_compile(tmp_path):
+    """include/bmt_hip.h is the boundary: it must compile as C99 and as C++ on its own, and the pybind11 forwarding
+    module that INTEGRATION.md shows a maintainer (the replacement for csrc/bind.cpp:3-35) must compile against it as
+    written, and link against the library."""
+    import subprocess
+    import sysconfig
+    import pybind11
+    import bmtrain_amd.C as C
+    include = os.path.join(ROOT, "include")
+    c_file = tmp_path / "uses_header.c"
+    c_file.write_text('#include "bmt_hip.h"\nint main(void) { return is_bf16_supported() == 1 ? 0 : 1; }\n')
+    lib_dir = os.path.dirname(C.LIBRARY_PATH)
+    exe = tmp_path / "uses_header"
+    subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-I", include, str(c_file), "-o", str(exe), "-L", lib_dir,
+                    "-lbmt_hip", "-Wl,-rpath," + lib_dir], check=True, capture_output=True)
+    assert subprocess.run([str(exe)]).returncode == 0
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    stub = re.search(r"```cpp\n(.*?)```", doc, flags=re.S).group(1)
+    assert "PYBIND11_MODULE(C, m)" in stub
+    cpp_file = tmp_path / "bind.cpp"
+    cpp_file.write_text(stub)
+    subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-Wall", "-Werror", "-I", include, "-I", pybind11.get_include(),
+                    "-I", sysconfig.get_paths()["include"], str(cpp_file)], check=True, capture_output=True)
