@@ -848,6 +848,12 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
     hipStream_t s = (hipStream_t)stream;
     if ((((uintptr_t)input | (uintptr_t)softmax) & 1u) != 0)
         return fail(-1, "cross_entropy_forward launcher: pointer is not 2-byte aligned");
+    // Not an in-place operation: the loss reads input[r, target[r]] after the row's softmax has been stored (in the
+    // reference as well, cross_entropy.cu:30-36), and the kernels here fetch parts of a row a second time.
+    {
+        const uintptr_t a = (uintptr_t)input, b = (uintptr_t)softmax, bytes = (uintptr_t)2 * (uintptr_t)m * (uintptr_t)n;
+        if (a < b + bytes && b < a + bytes) return fail(-1, "cross_entropy_forward launcher: softmax overlaps input");
+    }
     const int32_t nvec = n / 8;   // the most vectors a row can have
     if (same_vector_phase(input, softmax)) {
         // rows up to 32,768 elements live in the registers of their workgroup

@@ -120,6 +120,9 @@ BMT_API int to_bf16_from_fp32(int64_t n, const void *param_fp32, void *param_bf1
  *   softmax[r, :] = softmax(input[r, :]) rounded to the 16-bit type,
  *   output[r]     = target[r] != ignore_index ? logsumexp(input[r, :]) - input[r, target[r]] : 0.
  * m <= 0 or n <= 0 is a no-op (the reference would issue an invalid launch).
+ * softmax must not share memory with input: the loss is taken from input[r, target[r]] after
+ * the row's softmax has been stored (cross_entropy.cu:30-36 has the same order and gives an
+ * undefined loss in place); an overlapping pair is refused with status -1.
  */
 BMT_API int cross_entropy_forward_fp16_launcher(int32_t m, int32_t n, const void *input, const void *target,
                                         void *softmax, void *output, int32_t ignore_index, void *stream);

@@ -61,6 +61,11 @@ def test_argument_count_is_checked_and_degenerate_sizes_are_noops():
     C.cross_entropy_backward_inplace_bf16_launcher(4, 0, 0, 0, 0, -100, 0)
     with pytest.raises(RuntimeError, match="null pointer"):
         C.adam_cpu_fp16_launcher(4, 0, 0, 0, 0, 0, 0, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.0, 0.1, 0.001)
+    # refused on the host before any device call: a softmax output inside the logits (cross_entropy.cu:30-36 reads
+    # input[target] after the softmax row has been stored, so the forward is not an in-place operation there either)
+    for softmax in (0x10000, 0x10000 + 2 * 4 * 16 - 2, 0x10000 - 2 * 4 * 16 + 2):
+        with pytest.raises(RuntimeError, match="softmax overlaps input"):
+            C.cross_entropy_forward_bf16_launcher(4, 16, 0x10000, 0x40000, softmax, 0x50000, -100, 0)
 
 
 def test_header_is_plain_c_and_the_documented_bindings_compile(tmp_path):
