@@ -430,13 +430,34 @@ def full_model_side_measurements(torch, OF, p16, grad, p32, mom, var, iters=5):
     return out
 
 
+KERNEL_SOURCES = ("adam.hip", "cross_entropy.hip", "has_inf_nan.hip", "bmt_device.h", "bmt_host.h")
+
+
+def kernel_sources_digest():
+    """sha256 over the device sources: the measured traffic in profiles/ is tied to the kernels it was taken on."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "bmtrain_amd", "csrc", name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
+
+
 def load_measured_traffic():
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE); see profiles/."""
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE); see profiles/.  The file
+    records the digest of the kernel sources it was measured on; figures taken on other sources are not
+    reported (second element: where the figures come from, or why there are none)."""
     path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(path):
-        with open(path) as f:
-            return json.load(f)
-    return {}
+    if not os.path.exists(path):
+        return {}, "profiles/hbm_traffic.json is missing: traffic not reported"
+    with open(path) as f:
+        measured = json.load(f)
+    have, want = measured.get("_kernel_sources_sha256"), kernel_sources_digest()
+    if have != want:
+        return {}, ("profiles/hbm_traffic.json was measured on kernel sources with digest %s, the sources here have %s: "
+                    "traffic not reported" % (have, want))
+    return measured, ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command on these kernel sources "
+                      "(digest %s), read from profiles/hbm_traffic.json (not measured by this run)" % want)
 
 
 def main():
@@ -560,7 +581,7 @@ def main():
     ce_gbps = ce_bytes_per_row(classes) * rows / (ce_ms * 1e-3) / 1e9
     ce_fwd_gbps = (4 * classes + 8) * rows / (ms["ce_forward"] * 1e-3) / 1e9
     ce_bwd_gbps = (4 * classes + 8) * rows / (ms["ce_backward"] * 1e-3) / 1e9
-    traffic = load_measured_traffic()
+    traffic, traffic_source = load_measured_traffic()
 
     result = {
         "metric": "fused_adam_hbm_gbps_at_6.7b_params",
@@ -585,8 +606,7 @@ def main():
             "unit": "GB/s",
             "frac": round(adam_gbps / HBM_PEAK_GBPS, 4),
             "traffic": traffic.get("adam_stream_kernel", {}).get("bytes_per_launch") if not args.small else None,
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command, read from "
-                              "profiles/hbm_traffic.json (not measured by this run)",
+            "traffic_source": traffic_source,
             "algorithmic_bytes_per_launch": ADAM_BF16_BYTES * n,
             "ms_per_launch": round(ms["adam"], 4),
             **spread("adam"),
