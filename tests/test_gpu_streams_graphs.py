@@ -216,3 +216,48 @@ def test_entries_of_streams_with_work_in_flight_are_not_handed_on():
         torch.cuda.synchronize()
         for handle in handles:
             hip.hipStreamDestroy(handle)
+
+
+def test_host_threads_launching_at_once_on_their_own_streams():
+    """Six host threads (ctypes releases the interpreter lock for the call), each with a stream, buffers and state of
+    its own, run 12 whole steps at the same time: has_inf_nan, a resident-grid Adam launch, the long-row forward and
+    the resident in-place backward.  The library's only shared host state on this path is the per-device stream table
+    behind its mutex and a few cached device properties; every thread's result equals the one a single thread gets."""
+    import threading
+    n, rows, classes = (1 << 24) + 9, 300, 128256
+    x, t, soft0, loss0, go = _ce_inputs(rows, classes, 21)
+    want_state = _state(n, 5)
+    want_soft, want_loss = torch.empty_like(soft0), torch.empty_like(loss0)
+    want_flag = torch.zeros(1, dtype=torch.uint8, device="cuda")
+    for step in range(1, 13):
+        _step(*want_state, want_flag, x, t, want_soft, want_loss, go, step)
+    torch.cuda.synchronize()
+    threads, failures = [], []
+
+    def work(k):
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                state = _state(n, 5)
+                soft, loss = torch.empty_like(soft0), torch.empty_like(loss0)
+                flag = torch.zeros(1, dtype=torch.uint8, device="cuda")
+                for step in range(1, 13):
+                    _step(*state, flag, x, t, soft, loss, go, step)
+                stream.synchronize()
+                same = [torch.equal(a.view(torch.uint8), b.view(torch.uint8)) for a, b in zip(state, want_state)]
+                same += [torch.equal(soft.view(torch.int16), want_soft.view(torch.int16)), torch.equal(loss, want_loss),
+                         int(flag.item()) == 0]
+                if not all(same):
+                    failures.append((k, same))
+        except Exception as exc:                      # reported by the main thread
+            failures.append((k, repr(exc)))
+
+    for k in range(6):
+        threads.append(threading.Thread(target=work, args=(k,)))
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not any(th.is_alive() for th in threads)
+    assert failures == []
