@@ -647,22 +647,31 @@ constexpr int kFlatStreamThreads = 256;
 constexpr int kFlatStreamVecs = 4;                    // vectors per lane and tile
 constexpr int kFlatCounters = 8;
 constexpr int kFlatSlots = 256;
-constexpr int64_t kFlatStreamMinVec = (int64_t)1 << 22;       // 64 MiB
+// Smallest array (in 16-byte vectors) that runs as the resident grid: 2^27 elements, 256 MiB.  Measured against one
+// workgroup per tile, launches back to back on rows of 16,384 bf16 elements (% of peak, resident / per tile):
+// 2^25 elements 66.6 / 73.5, 2^26 76.3 / 79.3, 2^27 81.4 / 81.8, 2^28 83.1 / 82.4, 2^29 83.8 / 81.6, 2^30 (8,192 x 128,256)
+// 83.7 / 78; fp16 rows of 32,000: 6.6e7 elements 76.0 / 79.0, 1.3e8 81.2 / 81.6, 5.2e8 84.0 / 81.
+constexpr int64_t kFlatStreamMinVec = (int64_t)1 << 24;
 constexpr int32_t kFlatStreamMinRow = kFlatStreamThreads * kFlatStreamVecs * 8;
 // counter c of slot s: word c * 1024 + s * 4 (the counters of one launch sit 4 KiB apart); word s * 4 + 1 counts the
 // workgroups of the running launch that have left
 static __device__ __align__(256) uint32_t flat_tickets[kFlatCounters * 1024];
 
-__global__ void ce_flat_reset_kernel(uint32_t *tickets, uint32_t first_ticket) {
-    if (threadIdx.x < kFlatCounters) tickets[threadIdx.x * 1024] = first_ticket;
-    if (threadIdx.x == kFlatCounters) tickets[1] = 0u;
-}
-// The last workgroup to leave a launch writes the launch's number into the slot's word of pinned host memory:
-// from then on nothing draws from the slot's counters, and the host may hand the slot to another stream.
+// Counters start at zero (the array is zero when the library is loaded) and a launch leaves them at zero: every
+// workgroup has received its last ticket before it leaves (it waits for it), so when the last one leaves nothing
+// is drawing any more; that workgroup puts the eight counters and the count of leavers back to zero and then
+// writes the launch's number into the slot's word of pinned host memory (a release, so that the zeros are in
+// memory first): from then on the host may hand the slot to another stream.  No launch in front is needed.
 __device__ __forceinline__ void flat_leave(uint32_t *tickets, uint32_t *done_word, uint32_t launch_number) {
     if (threadIdx.x == 0) {
         const uint32_t left = __hip_atomic_fetch_add(tickets + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (left + 1 == gridDim.x) __hip_atomic_store(done_word, launch_number, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        if (left + 1 == gridDim.x) {
+#pragma unroll
+            for (int c = 0; c < kFlatCounters; c++)
+                __hip_atomic_store(tickets + c * 1024, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(tickets + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(done_word, launch_number, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
     }
 }
 
@@ -687,6 +696,7 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
     uint32_t *counter = tickets + which * 1024;
     const int64_t first = (int64_t)q * kFlatCounters + which;
     int64_t ahead = (int64_t)(q + (gridDim.x >> 3)) * kFlatCounters + which;
+    const uint32_t drawn_base = 2u * (gridDim.x >> 3);      // the first two tiles of a workgroup follow from its number
     if (first >= ntiles) { flat_leave(tickets, done_word, launch_number); return; }
     uint32_t drawn = 0;
     if (threadIdx.x == 0) stream_draw(drawn, counter);
@@ -738,7 +748,7 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
         asm volatile("s_waitcnt vmcnt(4)" : "+v"(cur.w[0]), "+v"(cur.w[1]), "+v"(cur.w[2]), "+v"(cur.w[3]), "+v"(drawn));
         if (threadIdx.x == 0) handed[slot] = drawn;
         __syncthreads();
-        ahead = (int64_t)handed[slot] * kFlatCounters + which;
+        ahead = (int64_t)(handed[slot] + drawn_base) * kFlatCounters + which;
         if (threadIdx.x == 0) stream_draw(drawn, counter);
         finish(cur);
         return tile;
@@ -992,7 +1002,6 @@ static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void 
                 const int cus = device_cu_count();
                 const unsigned grid = (unsigned)(cus >= 64 ? cus / 64 * 64 : 64);      // 8 XCDs x 8 counters
                 const int64_t per_tile = (int64_t)kFlatStreamThreads * kFlatStreamVecs;
-                hipLaunchKernelGGL(ce_flat_reset_kernel, dim3(1), dim3(64), 0, s, tickets, 2 * (grid / kFlatCounters));
                 hipLaunchKernelGGL((ce_flat_stream_kernel<T, OP>), dim3(grid), dim3(kFlatStreamThreads), 0, s, n, total_vec,
                                    (total_vec + per_tile - 1) / per_tile, (u32x4 *)x, (const float *)row_a, (const float *)row_b,
                                    (const int32_t *)target, tickets, fl.done_word, fl.number);

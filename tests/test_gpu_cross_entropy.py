@@ -221,12 +221,12 @@ def test_sumexp_and_softmax_inplace(name, dtype):
 
 @pytest.mark.parametrize("name,dtype", DTYPES)
 def test_elementwise_kernels_on_a_large_array(name, dtype):
-    """Arrays of 2^25 elements or more with rows of 8,192 or more run as a resident grid whose tiles (8,192
-    elements) straddle rows and whose last tile is ragged: 1,049 rows of 32,008.  Backward is bit-exact on identical
+    """Arrays of 2^27 elements or more with rows of 8,192 or more run as a resident grid whose tiles (8,192
+    elements) straddle rows and whose last tile is ragged: 4,197 rows of 32,008.  Backward is bit-exact on identical
     input, the in-place softmax within one unit in the last place; two launches on two streams at once use separate
     ticket counters; the words behind the array stay as they were."""
-    m, n = 1049, 32008
-    assert m * n >= 1 << 25 and (m * n // 8) % 1024 != 0 and n % 8192 != 0
+    m, n = 4197, 32008
+    assert m * n >= 1 << 27 and (m * n // 8) % 1024 != 0 and n % 8192 != 0
     x, t = _case(m, n, dtype, seed=77)
     soft, _ = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
     v = (torch.rand(m, generator=torch.Generator().manual_seed(5)) * 32768.0 / m).float()
@@ -266,7 +266,7 @@ def test_elementwise_kernels_on_more_streams_than_the_library_keeps_counters_for
     """The resident grid keeps its ticket counters per stream, for up to 256 streams of a device; a launch on a further
     stream gets the table entry of a stream whose last launch has completed, or takes the kernel that needs no
     counters.  260 streams, one launch each, same bits everywhere."""
-    m, n = 1049, 32008
+    m, n = 4197, 32008
     x, t = _case(m, n, torch.bfloat16, seed=78)
     soft, _ = oracle.ce_forward(bits16(x), t.numpy(), -100, "bf16")
     v = torch.full((m,), 1.0 / m)

@@ -100,7 +100,7 @@ def test_large_in_place_cross_entropy_kernels_captured_in_a_graph():
     """On a capturing stream the element-wise cross-entropy kernels of large arrays do without the library's ticket
     counters (a graph may be replayed on any stream, also on two at once); eager launches and replays give the same
     bits, replay after replay, with eager launches between them."""
-    rows, classes = 1049, 32008                         # 2^25 elements or more: the resident grid when launched eagerly
+    rows, classes = 4197, 32008                         # 2^27 elements or more: the resident grid when launched eagerly
     x, t, soft, loss, go = _ce_inputs(rows, classes, 9)
     LF.cross_entropy_forward(rows, classes, x, t, soft, loss, -100)
     eager = soft.clone()
@@ -145,7 +145,7 @@ def test_a_process_that_recycles_streams_keeps_the_resident_kernel():
     stream whose last launch has completed is handed on — and every checked result equals the first one."""
     from bmtrain_amd import C
     hip, ctypes = _runtime()
-    rows, classes = 1049, 32008
+    rows, classes = 4197, 32008
     x, t, soft, loss, go = _ce_inputs(rows, classes, 11)
     LF.cross_entropy_forward(rows, classes, x, t, soft, loss, -100)
     expect = soft.clone()
@@ -188,7 +188,7 @@ def test_entries_of_streams_with_work_in_flight_are_not_handed_on():
     kernel without counters), no two running launches may share counters — every buffer comes out exact."""
     from bmtrain_amd import C
     hip, ctypes = _runtime()
-    rows, classes = 1049, 32008
+    rows, classes = 4197, 32008
     x, t, soft, loss, go = _ce_inputs(rows, classes, 12)
     LF.cross_entropy_forward(rows, classes, x, t, soft, loss, -100)
     expect = soft.clone()
@@ -224,7 +224,7 @@ def test_host_threads_launching_at_once_on_their_own_streams():
     the resident in-place backward.  The library's only shared host state on this path is the per-device stream table
     behind its mutex and a few cached device properties; every thread's result equals the one a single thread gets."""
     import threading
-    n, rows, classes = (1 << 24) + 9, 300, 128256
+    n, rows, classes = (1 << 24) + 9, 1100, 128256
     x, t, soft0, loss0, go = _ce_inputs(rows, classes, 21)
     want_state = _state(n, 5)
     want_soft, want_loss = torch.empty_like(soft0), torch.empty_like(loss0)
