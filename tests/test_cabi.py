@@ -69,9 +69,9 @@ def test_argument_count_is_checked_and_degenerate_sizes_are_noops():
 
 
 def test_header_is_plain_c_and_the_documented_bindings_compile(tmp_path):
-    """include/bmt_hip.h is the boundary: it must compile as C99 and as C++ on its own, and the pybind11 forwarding
-    module that INTEGRATION.md shows a maintainer (the replacement for csrc/bind.cpp:3-35) must compile against it as
-    written, and link against the library."""
+    """include/bmt_hip.h is the boundary: it must compile as C99 on its own and link against the library, and the
+    pybind11 forwarding module that the integration guide shows a maintainer of the reference (the replacement for
+    csrc/bind.cpp:3-35, the guide's one C++ listing) must compile against the header exactly as printed there."""
     import subprocess
     import sysconfig
     import pybind11
