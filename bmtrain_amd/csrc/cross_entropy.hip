@@ -332,11 +332,13 @@ __global__ __launch_bounds__(kSmallThreads) void ce_forward_small_kernel(
 // Fine-grained load/compute interleaving in both sweeps lets the 32 waves of a CU hide each
 // other's latencies, which a whole-row-resident scheme with one or two workgroups per CU cannot.
 //
-// XR > 0 (rows of more than 12,288 vectors) keeps three more chunks: one in what is left of the CU's LDS — two
+// XR > 0 (rows of more than 10,240 vectors) keeps three more chunks: one in what is left of the CU's LDS — two
 // workgroups share 160 KiB, so all lanes but the last 16 find room for a fifth vector — and the two after it in
 // registers (58 VGPRs), and issues the four loads of the register part before it folds the first of them.  Together
 // 0.8 % at 128,256 classes (0.7597 -> 0.7529 ms, nine alternating rounds in one process); on rows that have no
-// dropped part the same code is 2 % slower, hence the condition.  Chunks are folded into the running sums two at a
+// dropped part the same code is 2 % slower, and so it is on rows of 9 or 10 chunks (8,192 x 81,920: 0.4575 against
+// 0.4511 ms); from 11 chunks on it is ahead (90,112: 0.5230 against 0.5327; 98,304: 0.5761 against 0.6067), hence the
+// condition.  Chunks are folded into the running sums two at a
 // time in row order either way, so the results do not depend on RK / LK / XR.
 template <typename T, int RK, int LK, int XR>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void ce_forward_retain_kernel(
@@ -884,8 +886,8 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
         else if (nvec <= 4096) BMT_CE_ROW(1024, 4);
         // up to 65,536 elements: 4 vectors per lane in registers, the rest in LDS, two workgroups per CU
         else if (nvec <= 6144) BMT_CE_RETAIN(6, 2, 4, 0);
-        // up to 98,304 elements: 8 vectors per lane kept, the rest fetched twice
-        else if (nvec <= 12288) BMT_CE_RETAIN(2 * ((nvec + 2047) / 2048), 4, 4, 0);
+        // up to 81,920 elements: 8 vectors per lane kept, the rest fetched twice
+        else if (nvec <= 10240) BMT_CE_RETAIN(2 * ((nvec + 2047) / 2048), 4, 4, 0);
         // longer rows: 11 vectors per lane kept (all but 16 lanes)
         else BMT_CE_RETAIN(2 * ((nvec + 2047) / 2048), 4, 4, 2);
     } else {

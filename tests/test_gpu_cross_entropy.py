@@ -38,7 +38,7 @@ def _forward_gpu(x, t, ignore=-100):
 # are not multiples of 8 (rows then start at every 2-byte offset in turn) in each of them
 WIDTHS = [1, 2, 3, 7, 8, 9, 10, 15, 16, 17, 90, 100, 512, 513, 520, 1000, 1001, 1024, 1500, 2048, 2056, 4096, 4097, 6100,
           8192, 8200, 10240, 12288, 12295, 16384, 20001, 30000, 32000, 32001, 32768, 32775, 49151, 50257, 50264, 65535,
-          65536, 65544, 98304, 100000, 100003, 128256, 128257, 131072, 131079, 131080, 151936, 151937, 256000, 300001]
+          65536, 65544, 81920, 81928, 90001, 98304, 100000, 100003, 128256, 128257, 131072, 131079, 131080, 151936, 151937, 256000, 300001]
 
 
 @pytest.mark.parametrize("name,dtype", DTYPES)
