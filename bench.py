@@ -296,13 +296,43 @@ def other_workloads(torch, dev, LF, OF, iters=20):
     out["ce_fp16_16384x32000_fwd_bwd"] = entry(stats, ce_bytes_per_row(classes) * rows, rows_per_s=round(rows / (stats[0] * 1e-3), 1))
     out["ce_fp16_16384x32000_forward"] = entry(
         timed(lambda: LF.cross_entropy_forward(rows, classes, x, t, soft, loss, -100)), (4 * classes + 8) * rows)
-    del x, soft
+    del soft
+
+    # the loss module around the kernels (bmtrain/loss/cross_entropy.py:216-260): output allocations, the ignore mask,
+    # the mean over valid rows and autograd, on top of the two launches; reported beside the kernels, outside the roofline
+    import bmtrain_amd as bmt
+    loss_fn = bmt.loss.FusedCrossEntropy(ignore_index=-100)
+
+    def module_step(logits, targets):
+        logits.grad = None
+        loss_fn(logits, targets).backward()
+
+    t64 = t.long()
+    x.requires_grad_(True)
+    stats = timed(lambda: module_step(x, t64))
+    out["ce_fp16_16384x32000_module_fwd_bwd"] = {
+        "ms": round(stats[0], 4), "ms_median": round(stats[1], 4), "ms_min": round(stats[2], 4),
+        "rows_per_s": round(rows / (stats[0] * 1e-3), 1),
+        "what": "FusedCrossEntropy(ignore_index=-100)(x, t).backward(): the two kernels plus allocation of the 1 GB softmax / "
+                "gradient tensor, the int32 cast of the targets, mask, mean and autograd"}
+    x.grad = None
+    del x, t64
     torch.cuda.empty_cache()
 
     # the two row helpers of the vocabulary-parallel loss, bf16, 8,192 rows x 128,256 classes
     rows, classes = 8192, 128256
     x = torch.empty(rows, classes, dtype=torch.bfloat16, device=dev)
     fill_normal_(x.view(-1), 3.0, gen)
+    t64 = torch.randint(0, classes, (rows,), generator=gen, device=dev)
+    t64[::20] = -100
+    x.requires_grad_(True)
+    stats = timed(lambda: module_step(x, t64))
+    out["ce_bf16_8192x128256_module_fwd_bwd"] = {
+        "ms": round(stats[0], 4), "ms_median": round(stats[1], 4), "ms_min": round(stats[2], 4),
+        "rows_per_s": round(rows / (stats[0] * 1e-3), 1), "what": "as above, 2.1 GB softmax / gradient tensor"}
+    x.grad = None
+    x.requires_grad_(False)
+    del t64
     row_max = torch.full((rows,), 14.0, dtype=torch.float32, device=dev)
     row_sum = torch.full((rows,), 5e4, dtype=torch.float32, device=dev)
     out["fused_sumexp_bf16_8192x128256"] = entry(timed(lambda: LF.fused_sumexp(x, row_max)), (2 * classes + 8) * rows)
