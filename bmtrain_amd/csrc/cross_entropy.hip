@@ -87,9 +87,16 @@ __device__ __forceinline__ float row_loss(const uint16_t *row, int32_t n, int32_
 }
 
 // How one row splits into 16-byte vectors.  A row may start anywhere (rows of odd length start at
-// every 2-byte offset in turn): up to 7 elements before the first 16-byte boundary, whole
-// vectors, up to 7 elements after the last one.  The (at most 14) edge elements are handled by
-// the first lanes of the workgroup, one element each, next to their share of the vectors.
+// every 2-byte offset in turn): `head` elements before the first boundary, whole vectors, up to 7
+// elements after the last one.  The edge elements are handled by the first lanes of the workgroup,
+// one element each, next to their share of the vectors.
+//
+// The boundary is a 16-byte one (`align` = 8 elements, at most 14 edge elements) or, in the kernels with
+// 256 lanes or more, a 128-byte one (`align` = 64, at most 70 edge elements): a wave then loads and stores
+// whole 128-byte lines.  Rows whose length is not a multiple of 64 elements start off the line grid, and a
+// workgroup that reads such a row and then writes it reaches 66 % of peak with vectors placed from the first
+// 16-byte boundary and 72 % with vectors placed from the first line boundary (bare access pattern, rows of
+// 256 KB; aligned rows: 72 %).  The launcher says which rows use it and what it measures on the kernels.
 struct RowSpan {
     const uint16_t *row;   // first element of the row
     int32_t head;          // elements before the first vector
@@ -99,10 +106,10 @@ struct RowSpan {
         return lane < head ? lane : head + 8 * nvec + (lane - head);
     }
 };
-__device__ __forceinline__ RowSpan row_span(const uint16_t *x, int64_t row, int32_t n) {
+__device__ __forceinline__ RowSpan row_span(const uint16_t *x, int64_t row, int32_t n, uint32_t align = 8u) {
     RowSpan sp;
     sp.row = x + row * n;
-    sp.head = (int32_t)((8u - (uint32_t)(((uintptr_t)sp.row >> 1) & 7u)) & 7u);
+    sp.head = (int32_t)((align - (uint32_t)(((uintptr_t)sp.row >> 1) & (align - 1u))) & (align - 1u));
     if (sp.head > n) sp.head = n;
     sp.nvec = (n - sp.head) >> 3;
     sp.nedge = n - 8 * sp.nvec;
@@ -127,10 +134,10 @@ __device__ __forceinline__ int64_t xcd_contiguous_row(uint32_t b, uint32_t rows)
 template <typename T, int THREADS, int CHUNKS>
 __global__ __launch_bounds__(THREADS) void ce_forward_row_kernel(
     int32_t n, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
-    uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index) {
+    uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index, uint32_t align) {
     __shared__ float slots[2][THREADS / kWave];
     const int64_t row = THREADS == 1024 ? xcd_contiguous_row(blockIdx.x, gridDim.x) : (int64_t)blockIdx.x;
-    const RowSpan sp = row_span(x, row, n);
+    const RowSpan sp = row_span(x, row, n, THREADS >= 256 ? align : 8u);
     const int32_t nvec = sp.nvec;
     const u32x4 *xr = (const u32x4 *)(sp.row + sp.head);
     uint16_t *srow = softmax + row * n;
@@ -343,7 +350,7 @@ __global__ __launch_bounds__(kSmallThreads) void ce_forward_small_kernel(
 template <typename T, int RK, int LK, int XR>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) void ce_forward_retain_kernel(
     int32_t n, const uint16_t *__restrict__ x, const int32_t *__restrict__ target,
-    uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index, int32_t chunks) {
+    uint16_t *__restrict__ softmax, float *__restrict__ out, int32_t ignore_index, int32_t chunks, uint32_t align) {
     constexpr int THREADS = 1024;
     constexpr int GROUP = 2;
     static_assert(RK % GROUP == 0 && LK % GROUP == 0, "chunk counts must be even");   // and so is `chunks`
@@ -353,7 +360,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8, 8))) vo
     extern __shared__ u32x4 staged[];  // LK * 1024 vectors, and kPartialLanes more when XR > 0
     __shared__ float slots[2][THREADS / kWave];
     const int64_t row = blockIdx.x;
-    const RowSpan sp = row_span(x, row, n);
+    const RowSpan sp = row_span(x, row, n, align);
     const int32_t nvec = sp.nvec;
     const u32x4 *xr = (const u32x4 *)(sp.row + sp.head);
     uint16_t *srow = softmax + row * n;
@@ -823,7 +830,7 @@ static int flat_grid(int64_t work_items, int threads_times_unroll) {
 #define BMT_CE_ROW(THREADS, CHUNKS)                                                                                \
     hipLaunchKernelGGL((ce_forward_row_kernel<T, THREADS, CHUNKS>), dim3((unsigned)m), dim3(THREADS), 0, s, n,         \
                        (const uint16_t *)input, (const int32_t *)target, (uint16_t *)softmax, (float *)output,     \
-                       ignore_index)
+                       ignore_index, align)
 
 #define BMT_CE_SMALL(LANES)                                                                                       \
     do {                                                                                                           \
@@ -849,7 +856,7 @@ static int flat_grid(int64_t work_items, int threads_times_unroll) {
         }                                                                                                          \
         hipLaunchKernelGGL(kern, dim3((unsigned)m), dim3(1024), lds, s, n, (const uint16_t *)input,                \
                            (const int32_t *)target, (uint16_t *)softmax, (float *)output, ignore_index,            \
-                           (int32_t)(CHUNKS));                                                                     \
+                           (int32_t)(CHUNKS), align);                                                              \
     } while (0)
 
 template <typename T>
@@ -867,6 +874,13 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
         if (a < b + bytes && b < a + bytes) return fail(-1, "cross_entropy_forward launcher: softmax overlaps input");
     }
     const int32_t nvec = n / 8;   // the most vectors a row can have
+    // Rows of more than 16,384 elements: vectors are placed from the first 128-byte line boundary of a row where both
+    // arrays sit at the same offset from one (any two torch allocations do), else from the first 16-byte boundary.
+    // Measured on rows that start off the line grid (2^29 elements in all, ms with 16-byte / with 128-byte placement):
+    // 8,192 x 86,583: 0.529 / 0.472; 128,257: 0.812 / 0.750; 16,384 x 32,001: 0.354 / 0.337; 65,544: 0.421 / 0.386;
+    // 20,488: 0.372 / 0.356; 16,392: 0.372 / 0.369; shorter rows gain or lose up to 5 % either way (up to 70 elements
+    // of a row then go through the one-element path), 2,056: 0.109 / 0.125.  Rows on the line grid are not affected.
+    const uint32_t align = (nvec > 2048 && ((((uintptr_t)input) ^ ((uintptr_t)softmax)) & 127u) == 0) ? 64u : 8u;
     if (same_vector_phase(input, softmax)) {
         // rows up to 32,768 elements live in the registers of their workgroup
         // short rows: several rows per wave

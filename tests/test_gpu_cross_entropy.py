@@ -60,8 +60,13 @@ def test_forward_against_oracle(name, dtype, n):
     elif name == "fp16":
         allowed = 4e-4 if n <= 8192 else 1.5e-4
     else:
-        allowed = 1.5e-4          # a single row can reach 2e-4 when its sum lands close to a rounding boundary of many quotients
-    assert (bits16(softmax) != want_soft).sum() <= 3 + allowed * m * n
+        allowed = 1.5e-4
+    # The differing elements of a row move together with its sum: when the sum lands on the other side of an fp32
+    # rounding than the oracle's, the row's quotients that sit next to a 16-bit rounding boundary all flip.  Over 240
+    # rows per width and type the worst single row differs on 1.4e-3 of its elements (bf16; fp16 4e-4) while the mean
+    # stays at 1e-5 to 4e-5, so a sample of only nine long rows needs room for one such row on top of the rate.
+    one_unlucky_row = (1.5e-3 if name == "bf16" else 5e-4) * n
+    assert (bits16(softmax) != want_soft).sum() <= 3 + allowed * m * n + one_unlucky_row
     np.testing.assert_allclose(loss.cpu().numpy(), want_loss, rtol=2e-6, atol=2e-6)
     ref32 = torch.nn.functional.cross_entropy(x.float(), t.long(), ignore_index=-100, reduction="none").numpy()
     np.testing.assert_allclose(loss.cpu().numpy(), ref32, rtol=1e-3, atol=1e-6)
@@ -178,17 +183,18 @@ def test_special_rows(name, dtype, n):
 
 
 @pytest.mark.parametrize("name,dtype", DTYPES)
-@pytest.mark.parametrize("m,n", [(6, 1024), (5, 1001), (3, 50257), (2, 131075), (40, 5), (9, 8)])
+@pytest.mark.parametrize("m,n", [(6, 1024), (5, 1001), (3, 50257), (2, 131075), (3, 20488), (4, 86583), (40, 5), (9, 8)])
 def test_unaligned_bases(name, dtype, m, n):
-    """Arrays that start at any 2-byte offset: logits and softmax at the same offset from a 16-byte boundary
-    (vector kernels with a per-row split) and at different ones (element loads); nothing outside is written."""
+    """Arrays that start at any 2-byte offset: logits and softmax at the same offset from a 128-byte line (long rows:
+    vectors placed from each row's first line boundary), at the same offset from a 16-byte boundary only (vectors
+    placed from the first 16-byte boundary) and at different ones (element loads); nothing outside is written."""
     x, t = _case(m, n, dtype, seed=n + m)
     want_soft, want_loss = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
-    buf = torch.zeros(m * n + 16, dtype=dtype, device="cuda")
-    for off, soft_off in ((1, 1), (4, 4), (7, 7), (3, 11), (0, 8), (2, 5), (0, 1)):
+    buf = torch.zeros(m * n + 80, dtype=dtype, device="cuda")
+    for off, soft_off in ((1, 1), (4, 4), (7, 7), (63, 63), (0, 64), (9, 73), (3, 11), (0, 8), (24, 40), (2, 5), (0, 1)):
         xg = buf[off:off + m * n].view(m, n)
         xg.copy_(x)
-        soft_buf = torch.zeros(m * n + 16, dtype=dtype, device="cuda")
+        soft_buf = torch.zeros(m * n + 80, dtype=dtype, device="cuda")
         soft = soft_buf[soft_off:soft_off + m * n].view(m, n)
         out = torch.empty(m, dtype=torch.float32, device="cuda")
         F.cross_entropy_forward(m, n, xg, t.cuda(), soft, out, -100)
