@@ -360,7 +360,7 @@ __global__ __launch_bounds__(kAdamScalarThreads) void adam_fp16_scalar_kernel(
 // tail, given the addresses of the fp32 arrays (16-byte vectors) and the 16-bit
 // arrays (8-byte vectors).  Returns false when the arrays do not share one phase.
 static bool split_for_vectors(int64_t n, const uintptr_t *addr32, int n32, const uintptr_t *addr16, int n16,
-                              int64_t *head, int64_t *nvec) {
+                              int64_t resident_min_vec, int64_t *head, int64_t *nvec) {
     // Elements to skip until the address is vector-aligned; must agree across arrays.
     int64_t want = -1;
     for (int k = 0; k < n32; k++) {
@@ -374,6 +374,16 @@ static bool split_for_vectors(int64_t n, const uintptr_t *addr32, int n32, const
         if (want < 0) want = skip; else if (want != skip) return false;
     }
     if (want > n) want = n;
+    // Tiles are 4 KiB blocks of the fp32 arrays (the granularity at which HBM channels interleave) counted from the
+    // first group, so a body that starts off that grid makes every tile straddle two blocks: one transformer block
+    // stepped through views 8 elements into its buffers runs at 77.5 % of peak, 256 elements in at 81.5 %, 1,024
+    // elements in (on the grid again) at 84 %.  Calls that run as the resident grid therefore hand the elements up to
+    // the fp32 parameters' next 4 KiB boundary (at most 1,023) to the element kernel as well; the step to that boundary
+    // is the step to the next 16-byte boundary plus whole vectors, so it suits every array of the call.
+    // The one-tile kernel of shorter calls only needs whole lines and would pay for the extra launch (2^23 elements,
+    // 64 elements in: 72 % as it is, 67 % with the longer head).
+    const int64_t to_grid = (int64_t)(((4096 - (addr32[0] & 4095u)) & 4095u) / 4);     // = want modulo 4
+    if (to_grid > want && (n - to_grid) / 4 >= resident_min_vec) want = to_grid;
     *head = want;
     *nvec = (n - want) / 4;
     return true;
@@ -422,7 +432,7 @@ static hipError_t launch_bf16(int64_t n, float *p32, uint16_t *p16, const uint16
     uintptr_t a32[3] = {(uintptr_t)p32, (uintptr_t)m, (uintptr_t)v};
     uintptr_t a16[2] = {(uintptr_t)p16, (uintptr_t)g};
     int64_t head = 0, nvec = 0;
-    const bool vectorisable = split_for_vectors(n, a32, 3, a16, 2, &head, &nvec);
+    const bool vectorisable = split_for_vectors(n, a32, 3, a16, 2, kStreamMinVecBf16, &head, &nvec);
     return launch_split(
         n, vectorisable, head, nvec,
         [&](unsigned grid) {
@@ -452,7 +462,7 @@ static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16
     uintptr_t a32[2] = {(uintptr_t)p32, (uintptr_t)v};
     uintptr_t a16[3] = {(uintptr_t)p16, (uintptr_t)g, (uintptr_t)m};
     int64_t head = 0, nvec = 0;
-    const bool vectorisable = split_for_vectors(n, a32, 2, a16, 3, &head, &nvec);
+    const bool vectorisable = split_for_vectors(n, a32, 2, a16, 3, kStreamMinVecFp16, &head, &nvec);
     return launch_split(
         n, vectorisable, head, nvec,
         [&](unsigned grid) {

@@ -302,13 +302,17 @@ def test_one_transformer_block_flat_buffer():
 @pytest.mark.parametrize("flavour", ["bf16", "fp16"])
 @pytest.mark.parametrize("n,off", [((3 << 22) - 1, 0), ((3 << 22) + 2, 2), ((3 << 22) + 1024 * 7 + 5, 1), ((3 << 22) + 12, 3),
                                    ((1 << 24) - 1, 0), ((1 << 24) + 2, 2), ((1 << 24) + 1024 * 7 + 5, 1), ((1 << 24) + 4 * 2048 + 3, 0),
-                                   ((1 << 25) + 12345, 0), ((1 << 25) + 4096 * 3 + 1, 2), (3 * (1 << 24) + 4 * 1537, 3)])
+                                   ((1 << 25) + 12345, 0), ((1 << 25) + 4096 * 3 + 1, 2), (3 * (1 << 24) + 4 * 1537, 3),
+                                   ((1 << 24) + 77, 8), ((3 << 22) + 5000, 256), ((1 << 25) + 1, 1000), ((3 << 22) + 1023, 1),
+                                   ((3 << 22) + 1020, 4)])
 def test_around_the_launch_size_where_the_resident_grid_takes_over(flavour, n, off):
     """From 3 * 2^20 (bf16) or 2^22 (fp16) four-element groups on, a resident grid draws tiles of 256 groups from four
     counters kept in the 16-bit output (word 0 of the vectors nvec-1, nvec-513, nvec-1025, nvec-1537), whose real
     values a small kernel restores afterwards.  Whole-buffer comparison with the oracle just below and above both
     sizes, with unaligned heads and partial last tiles: every tile stepped exactly once, and the counters' places
-    hold their real values."""
+    hold their real values.  A resident launch starts its tiles at the fp32 parameters' next 4 KiB boundary and leaves
+    the up to 1,023 elements in front of it to the element kernel (offsets 1 to 1,000 below), unless that would take
+    the call below the size of a resident launch (the last two cases)."""
     dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
     mdt = torch.float16 if flavour == "fp16" else torch.float32
     scale = 4.0 if flavour == "fp16" else 1.0
@@ -318,7 +322,7 @@ def test_around_the_launch_size_where_the_resident_grid_takes_over(flavour, n, o
     v = (torch.randn(n, generator=gen) * 1e-6 * scale).abs()
     g = (torch.randn(n, generator=gen) * 1e-3 * scale).to(dt16)
     def place(t, fill=0):
-        buf = torch.full((n + 8,), fill, dtype=t.dtype, device="cuda")
+        buf = torch.full((n + 1032,), fill, dtype=t.dtype, device="cuda")
         buf[off:off + n] = t.cuda()
         return buf[off:off + n]
     pg, mg, vg, gg = place(p), place(m), place(v), place(g)
