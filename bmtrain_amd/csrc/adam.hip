@@ -109,14 +109,30 @@ __device__ __forceinline__ void st(T *p, T v) { __builtin_nontemporal_store(v, p
 constexpr int kAdamThreads = 1024;
 constexpr int kAdamUnroll = 1;
 
+// A call's elements in front of and behind its vector body (the arrays may start anywhere): lane t < head takes
+// element t - head, lane head + k takes the k-th element behind the body; indices count from the body's first element.
+// The first workgroup of the one-tile kernels steps them next to its tile, with the per-element routine that the
+// element kernels use, so such a call stays one launch.
+__device__ __forceinline__ int64_t edge_element(int64_t nvec, int32_t head) {
+    const int32_t t = (int32_t)threadIdx.x;
+    return t < head ? (int64_t)t - head : 4 * nvec + (t - head);
+}
+
 // Vector body, bf16.  `nvec` = number of 4-element groups; every pointer is aligned for its
 // vector type.  A tile is kAdamThreads * UNROLL groups; group u of a lane sits kAdamThreads groups
 // after group u-1, so each load instruction of a wave covers 64 consecutive vectors (1 KiB of fp32).
 template <int UNROLL>
 __global__ __launch_bounds__(kAdamThreads) void adam_bf16_vec_kernel(
     int64_t nvec, f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, const u32x2 *__restrict__ g16,
-    f32x4 *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h) {
+    f32x4 *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h, int32_t head, int32_t tail) {
     const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd;
+    if (blockIdx.x == 0 && (int)threadIdx.x < head + tail) {      // the elements around the vector body, one per lane
+        const int64_t e = edge_element(nvec, head);
+        float *p1 = (float *)p32 + e, *m1 = (float *)mom + e, *v1 = (float *)var + e;
+        float p = *p1, m = *m1, v = *v1;
+        adam_elem_unscaled(clip16<BFloat16>(BFloat16::to_f32(((const uint16_t *)g16)[e]), h.gcoef), m, v, p, h, omb1, omb2, lrwd);
+        *p1 = p; *m1 = m; *v1 = v; ((uint16_t *)p16)[e] = BFloat16::from_f32(p);
+    }
     const int64_t base = (int64_t)blockIdx.x * (kAdamThreads * UNROLL) + threadIdx.x;
     f32x4 p[UNROLL], m[UNROLL], v[UNROLL];
     u32x2 g[UNROLL];
@@ -143,8 +159,16 @@ __global__ __launch_bounds__(kAdamThreads) void adam_bf16_vec_kernel(
 template <int UNROLL>
 __global__ __launch_bounds__(kAdamThreads) void adam_fp16_vec_kernel(
     int64_t nvec, f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, const u32x2 *__restrict__ g16,
-    u32x2 *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h) {
+    u32x2 *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h, int32_t head, int32_t tail) {
     const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
+    if (blockIdx.x == 0 && (int)threadIdx.x < head + tail) {      // the elements around the vector body, one per lane
+        const int64_t e = edge_element(nvec, head);
+        float *p1 = (float *)p32 + e, *v1 = (float *)var + e;
+        uint16_t *m1 = (uint16_t *)mom + e;
+        float p = *p1, m = Half::to_f32(*m1), v = *v1;
+        adam_elem_scaled(clip16<Half>(Half::to_f32(((const uint16_t *)g16)[e]), h.gcoef), m, v, p, h, omb1, omb2, lrwd, eps_s);
+        *p1 = p; *m1 = Half::from_f32(m); *v1 = v; ((uint16_t *)p16)[e] = Half::from_f32(p);
+    }
     const int64_t base = (int64_t)blockIdx.x * (kAdamThreads * UNROLL) + threadIdx.x;
     f32x4 p[UNROLL], v[UNROLL];
     u32x2 g[UNROLL], mh[UNROLL];
@@ -356,6 +380,7 @@ __global__ __launch_bounds__(kAdamScalarThreads) void adam_fp16_scalar_kernel(
     }
 }
 
+constexpr int64_t kLineAlignMinVec = 4096;       // 16,384 elements: below that the head would be a visible share of the call
 // Splits [0, n) into a scalar head, a vector body of 4-element groups and a scalar
 // tail, given the addresses of the fp32 arrays (16-byte vectors) and the 16-bit
 // arrays (8-byte vectors).  Returns false when the arrays do not share one phase.
@@ -383,13 +408,19 @@ static bool split_for_vectors(int64_t n, const uintptr_t *addr32, int n32, const
     // The one-tile kernel of shorter calls only needs whole lines and would pay for the extra launch (2^23 elements,
     // 64 elements in: 72 % as it is, 67 % with the longer head).
     const int64_t to_grid = (int64_t)(((4096 - (addr32[0] & 4095u)) & 4095u) / 4);     // = want modulo 4
+    // Shorter calls start their body on a 256-byte boundary of the fp32 parameters (a 128-byte line of the 16-bit
+    // arrays; 2^23 elements reached through views 8 or 1,000 elements into their buffers: 65-67 % of peak as they
+    // are, 72 % on the lines); the up to 63 elements in front are stepped by the vector kernel's first workgroup.
+    const int64_t to_line = (int64_t)(((256 - (addr32[0] & 255u)) & 255u) / 4);        // = want modulo 4
     if (to_grid > want && (n - to_grid) / 4 >= resident_min_vec) want = to_grid;
+    else if (to_line > want && (n - to_line) / 4 >= kLineAlignMinVec) want = to_line;
     *head = want;
     *nvec = (n - want) / 4;
     return true;
 }
 
-// Launches the vector body over [head, head + 4 * nvec) and the element kernel over what is left.
+// Launches the vector body over [head, head + 4 * nvec) and, unless the vector launch has stepped them itself
+// (it says so), the element kernel over what is left.
 template <typename VecLaunch, typename ScalarLaunch>
 static hipError_t launch_split(int64_t n, bool vectorisable, int64_t head, int64_t nvec, const VecLaunch &vec,
                                const ScalarLaunch &scalar) {
@@ -403,9 +434,9 @@ static hipError_t launch_split(int64_t n, bool vectorisable, int64_t head, int64
         const int64_t tile = (int64_t)kAdamThreads * kAdamUnroll;
         const int64_t ntiles = (nvec + tile - 1) / tile;
         if (ntiles > 0x7FFFFFFF) return hipErrorInvalidValue;
-        vec((unsigned)ntiles);
+        const bool edges_done = vec((unsigned)ntiles, (int32_t)(head <= 1023 ? head : -1), (int32_t)(n - head - nvec * 4));
         hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
+        if (e != hipSuccess || edges_done) return e;
     }
     const int64_t tail_lo = head + nvec * 4;
     if (head > 0 || tail_lo < n) {
@@ -435,7 +466,7 @@ static hipError_t launch_bf16(int64_t n, float *p32, uint16_t *p16, const uint16
     const bool vectorisable = split_for_vectors(n, a32, 3, a16, 2, kStreamMinVecBf16, &head, &nvec);
     return launch_split(
         n, vectorisable, head, nvec,
-        [&](unsigned grid) {
+        [&](unsigned grid, int32_t head_elements, int32_t tail_elements) -> bool {
             u32x2 *out16 = (u32x2 *)(p16 + head);
             if (nvec >= kStreamMinVecBf16) {
                 const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
@@ -445,11 +476,13 @@ static hipError_t launch_bf16(int64_t n, float *p32, uint16_t *p16, const uint16
                                    (f32x4 *)(v + head), h);
                 hipLaunchKernelGGL((adam_stream_finish_kernel<BFloat16>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
                                    out16, nvec);
-            } else {
-                hipLaunchKernelGGL((adam_bf16_vec_kernel<kAdamUnroll>), dim3(grid), dim3(kAdamThreads), 0, s, nvec,
-                                   (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (f32x4 *)(m + head),
-                                   (f32x4 *)(v + head), h);
+                return false;
             }
+            const bool with_edges = head_elements >= 0 && head_elements + tail_elements <= kAdamThreads;
+            hipLaunchKernelGGL((adam_bf16_vec_kernel<kAdamUnroll>), dim3(grid), dim3(kAdamThreads), 0, s, nvec,
+                               (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (f32x4 *)(m + head),
+                               (f32x4 *)(v + head), h, with_edges ? head_elements : 0, with_edges ? tail_elements : 0);
+            return with_edges;
         },
         [&](unsigned grid, int64_t lo0, int64_t hi0, int64_t lo1, int64_t hi1) {
             hipLaunchKernelGGL(adam_bf16_scalar_kernel, dim3(grid), dim3(kAdamScalarThreads), 0, s, lo0, hi0, lo1, hi1,
@@ -465,7 +498,7 @@ static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16
     const bool vectorisable = split_for_vectors(n, a32, 2, a16, 3, kStreamMinVecFp16, &head, &nvec);
     return launch_split(
         n, vectorisable, head, nvec,
-        [&](unsigned grid) {
+        [&](unsigned grid, int32_t head_elements, int32_t tail_elements) -> bool {
             u32x2 *out16 = (u32x2 *)(p16 + head);
             if (nvec >= kStreamMinVecFp16) {
                 const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
@@ -475,11 +508,13 @@ static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16
                                    (f32x4 *)(v + head), h);
                 hipLaunchKernelGGL((adam_stream_finish_kernel<Half>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
                                    out16, nvec);
-            } else {
-                hipLaunchKernelGGL((adam_fp16_vec_kernel<kAdamUnroll>), dim3(grid), dim3(kAdamThreads), 0, s, nvec,
-                                   (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
-                                   (f32x4 *)(v + head), h);
+                return false;
             }
+            const bool with_edges = head_elements >= 0 && head_elements + tail_elements <= kAdamThreads;
+            hipLaunchKernelGGL((adam_fp16_vec_kernel<kAdamUnroll>), dim3(grid), dim3(kAdamThreads), 0, s, nvec,
+                               (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
+                               (f32x4 *)(v + head), h, with_edges ? head_elements : 0, with_edges ? tail_elements : 0);
+            return with_edges;
         },
         [&](unsigned grid, int64_t lo0, int64_t hi0, int64_t lo1, int64_t hi1) {
             hipLaunchKernelGGL(adam_fp16_scalar_kernel, dim3(grid), dim3(kAdamScalarThreads), 0, s, lo0, hi0, lo1, hi1,
