@@ -249,6 +249,13 @@ def other_workloads(torch, dev, LF, OF, iters=20):
                      ("adam_bf16_one_tensor_11008x4096", 11008 * 4096)):
         out[label] = entry(timed_batches(torch, lambda: OF.adam_bf16(p32[:k], p16[:k], grad[:k], mom[:k], var[:k], 0.9, 0.999, 1e-8, 1e-3,
                                                                      1.0, 0.01, 100), 64, per_batch=16), ADAM_BF16_BYTES * k, elements=k)
+    # the same through views that start off every grid (parameters anywhere inside a flat buffer): 1,001 elements in
+    for label, k in (("adam_bf16_one_tensor_2^23_view_1001_elements_in", 1 << 23),
+                     ("adam_bf16_one_tensor_45M_view_1001_elements_in", 11008 * 4096)):
+        lo = 1001
+        out[label] = entry(timed_batches(torch, lambda: OF.adam_bf16(p32[lo:lo + k], p16[lo:lo + k], grad[lo:lo + k], mom[lo:lo + k],
+                                                                     var[lo:lo + k], 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 100),
+                                         64, per_batch=16), ADAM_BF16_BYTES * k, elements=k)
     del p16, grad, p32, mom, var
     torch.cuda.empty_cache()
     # the fp16 flavour (24 B / element: the first moment is a 16-bit array, kept multiplied by the loss scale), on buffers of its own
