@@ -327,20 +327,14 @@ def other_workloads(torch, dev, LF, OF, iters=20):
     torch.cuda.empty_cache()
 
     # a vocabulary that is not a multiple of 64 (86,583 classes): every row starts at another offset from the 128-byte lines
-    rows, classes = 8192, 86583
+    # (the forward only: the backward works on the flat array and never sees rows)
+    rows, classes = 6144, 86583
     x = torch.empty(rows, classes, dtype=torch.bfloat16, device=dev)
     fill_normal_(x.view(-1), 3.0, gen)
     t = torch.randint(0, classes, (rows,), generator=gen, device=dev, dtype=torch.int32)
     soft = torch.empty_like(x)
     loss = torch.empty(rows, dtype=torch.float32, device=dev)
-    go = torch.full((rows,), 1.0 / rows, device=dev)
-
-    def fwd_bwd_odd():
-        LF.cross_entropy_forward(rows, classes, x, t, soft, loss, -100)
-        LF.cross_entropy_backward_inplace(rows, classes, go, t, soft, -100)
-    stats = timed(fwd_bwd_odd)
-    out["ce_bf16_8192x86583_fwd_bwd"] = entry(stats, ce_bytes_per_row(classes) * rows, rows_per_s=round(rows / (stats[0] * 1e-3), 1))
-    out["ce_bf16_8192x86583_forward"] = entry(
+    out["ce_bf16_6144x86583_forward"] = entry(
         timed(lambda: LF.cross_entropy_forward(rows, classes, x, t, soft, loss, -100)), (4 * classes + 8) * rows)
     del x, soft, t
     torch.cuda.empty_cache()
