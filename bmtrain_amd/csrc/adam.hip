@@ -221,19 +221,24 @@ __global__ __launch_bounds__(kAdamThreads) void adam_fp16_vec_kernel(
 // registers for two more cycles, and the compiler, which pads that hazard itself for stores it
 // emits, does not see through an asm statement.
 //
-// The four counters live in the caller's 16-bit parameter output (nothing else is writable
-// without a workspace argument): word 0 of the 8-byte vectors nvec-1, nvec-513, nvec-1025 and
-// nvec-1537.  A one-workgroup kernel in front zeroes them; the lanes that own those four groups
-// step them like any other but do not store their 16-bit result; a one-workgroup kernel behind
-// derives those four vectors from the fp32 parameters just written (the 16-bit copy is by
-// definition the rounded fp32 value).  All three run on the caller's stream, so the ordering
-// between the zeroing, the atomics (performed in memory, beyond the per-XCD L2s) and the final
-// plain stores is that of kernel boundaries.
+// Where the four counters live depends on the stream.  A stream that has an entry in the library's
+// stream table (stream_slot_for, bmt_host.h) uses that entry's counters in the library's own device
+// array: one kernel, the last workgroup to leave puts the counters back to zero.  Otherwise (a stream
+// under graph capture, the per-thread default stream, a busy table; the multi-tensor kernel always)
+// they live in the caller's 16-bit parameter output, the only memory of the call that the step never
+// reads: word 0 of the 8-byte vectors nvec-1, nvec-513, nvec-1025 and nvec-1537.  A one-workgroup
+// kernel in front zeroes them; the lanes that own those four groups step them like any other but do
+// not store their 16-bit result; a one-workgroup kernel behind derives those four vectors from the
+// fp32 parameters just written (the 16-bit copy is by definition the rounded fp32 value).  All three
+// run on the caller's stream, so the ordering between the zeroing, the atomics (performed in memory,
+// beyond the per-XCD L2s) and the final plain stores is that of kernel boundaries.  Measured, slot
+// against output-hosted counters: bf16 12.6 M elements 73.6 / 72.3 % of peak, 16.8 M 77.6 / 76.1,
+// 45 M 82.4 / 81.8, from 131 M on the same; 3.5 against 9.2 us of host time per call.
 constexpr int kStreamThreads = 256;
 constexpr int kStreamCounters = 4;
 constexpr int64_t kStreamCounterStride = 512;            // in 8-byte vectors: 4 KiB
 // Smallest launch (in 4-element groups) that runs as the resident grid, where it overtakes one workgroup per
-// tile (two more one-workgroup launches per call, about 9 us).  Measured per flavour, launches back to back:
+// tile.  Measured per flavour with the counters in the 16-bit output, launches back to back:
 //   bf16   10.5 M elements: 71 % of peak either way;  12.6 M: 74.3 against 71.7;  14.7 M: 76.2 against 73.9;
 //          8.4 M: 70.3 against 74.0;  4.2 M: 58.7 against 70.7
 //   fp16   12.6 M: 70.2 against 73.2;  16.8 M: 73.2 against 73.9;  202 M: 80.0 against 72.8
@@ -244,10 +249,10 @@ __device__ __forceinline__ bool holds_stream_counter(int64_t i, int64_t nvec) {
     const int64_t d = nvec - 1 - i;
     return (d & (kStreamCounterStride - 1)) == 0 && d < kStreamCounters * kStreamCounterStride;
 }
-// Every workgroup starts on two tiles it can name itself (see stream_first_tickets), so the counters
-// start at twice the number of workgroups that share a counter.
-__global__ void adam_stream_reset_kernel(u32x2 *p16, int64_t nvec, uint32_t first_ticket) {
-    if (threadIdx.x < kStreamCounters) p16[nvec - 1 - threadIdx.x * kStreamCounterStride] = u32x2{first_ticket, 0u};
+// Every workgroup starts on two tiles it can name itself (see stream_first_tickets), so a ticket drawn from a
+// counter (which starts at zero) counts from twice the number of workgroups that share the counter.
+__global__ void adam_stream_reset_kernel(u32x2 *p16, int64_t nvec) {
+    if (threadIdx.x < kStreamCounters) p16[nvec - 1 - threadIdx.x * kStreamCounterStride] = u32x2{0u, 0u};
 }
 // The grid of the resident kernels: one workgroup per compute unit, rounded down to a multiple of 32
 // (8 XCDs x 4 counters), at least 32.
@@ -287,20 +292,28 @@ struct StreamSet {
     bool ok;        // the group exists
 };
 
-template <bool FP16>
+// SLOT: the counters are a slot of the library's own array (stream_slot_for) instead of places in the 16-bit output;
+// every group then stores its 16-bit result, nothing runs in front of or behind the kernel, and the last workgroup to
+// leave puts the slot back (stream_slot_leave).
+template <bool FP16, bool SLOT>
 __global__ __launch_bounds__(kStreamThreads) void adam_stream_kernel(
     int64_t nvec, int64_t ntiles, f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, const u32x2 *__restrict__ g16,
-    typename MomentVec<FP16>::type *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h) {
+    typename MomentVec<FP16>::type *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h, uint32_t *__restrict__ slot,
+    uint32_t *__restrict__ done_word, uint32_t launch_number) {
     typedef StreamSet<FP16> Set;
     const float omb1 = 1.0f - h.b1, omb2 = 1.0f - h.b2, lrwd = h.lr * h.wd, eps_s = h.eps * h.scale;
     __shared__ uint32_t handed[2];
     int which;
     uint32_t t0, t1;
     stream_first_tickets(which, t0, t1);
-    uint32_t *counter = (uint32_t *)(p16 + (nvec - 1 - which * kStreamCounterStride));
+    uint32_t *counter = SLOT ? slot + which * 1024 : (uint32_t *)(p16 + (nvec - 1 - which * kStreamCounterStride));
+    const uint32_t drawn_base = gridDim.x >> 1;                       // two tickets per workgroup are taken already
     const int64_t first = (int64_t)t0 * kStreamCounters + which;
     int64_t ahead = (int64_t)t1 * kStreamCounters + which;            // the tile after the one in flight
-    if (first >= ntiles) return;
+    if (first >= ntiles) {
+        if (SLOT) stream_slot_leave(slot, done_word, launch_number);
+        return;
+    }
     uint32_t drawn = 0;                                               // lane 0: ticket on its way
     if (threadIdx.x == 0) stream_draw(drawn, counter);
 
@@ -328,17 +341,17 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_kernel(
         stream_store(p32 + s.i, s.p);
         stream_store(mom + s.i, s.m);
         stream_store(var + s.i, s.v);
-        if (!holds_stream_counter(s.i, nvec)) stream_store(p16 + s.i, o);
+        if (SLOT || !holds_stream_counter(s.i, nvec)) stream_store(p16 + s.i, o);
     };
     // One stage: the loads of the tile after `cur` go out, then `cur` is computed and stored.
     // Returns the tile whose loads went out.
-    auto stage = [&](Set &cur, Set &next, int slot) -> int64_t {
+    auto stage = [&](Set &cur, Set &next, int turn) -> int64_t {
         const int64_t tile = ahead;
         issue(next, tile);
         asm volatile("s_waitcnt vmcnt(4)" : "+v"(cur.g), "+v"(cur.p), "+v"(cur.m), "+v"(cur.v), "+v"(drawn));
-        if (threadIdx.x == 0) handed[slot] = drawn;
+        if (threadIdx.x == 0) handed[turn] = drawn;
         __syncthreads();
-        ahead = (int64_t)handed[slot] * kStreamCounters + which;
+        ahead = (int64_t)(handed[turn] + drawn_base) * kStreamCounters + which;
         if (threadIdx.x == 0) stream_draw(drawn, counter);
         finish(cur);
         return tile;
@@ -350,6 +363,7 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_kernel(
         if (stage(b, a, 1) >= ntiles) break;
     }
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");   // loads of the tile nobody owns, the last ticket
+    if (SLOT) stream_slot_leave(slot, done_word, launch_number);
 }
 
 constexpr int kAdamScalarThreads = 256;
@@ -470,10 +484,17 @@ static hipError_t launch_bf16(int64_t n, float *p32, uint16_t *p16, const uint16
             u32x2 *out16 = (u32x2 *)(p16 + head);
             if (nvec >= kStreamMinVecBf16) {
                 const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
-                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec, stream_grid() / 2);
-                hipLaunchKernelGGL((adam_stream_kernel<false>), dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
+                StreamSlot slot;
+                if (stream_slot_for(s, &slot, false)) {
+                    hipLaunchKernelGGL((adam_stream_kernel<false, true>), dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
+                                       ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (f32x4 *)(m + head),
+                                       (f32x4 *)(v + head), h, slot.tickets, slot.done_word, slot.number);
+                    return false;
+                }
+                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec);
+                hipLaunchKernelGGL((adam_stream_kernel<false, false>), dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
                                    ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (f32x4 *)(m + head),
-                                   (f32x4 *)(v + head), h);
+                                   (f32x4 *)(v + head), h, (uint32_t *)nullptr, (uint32_t *)nullptr, 0u);
                 hipLaunchKernelGGL((adam_stream_finish_kernel<BFloat16>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
                                    out16, nvec);
                 return false;
@@ -502,10 +523,17 @@ static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16
             u32x2 *out16 = (u32x2 *)(p16 + head);
             if (nvec >= kStreamMinVecFp16) {
                 const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
-                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec, stream_grid(true) / 2);
-                hipLaunchKernelGGL((adam_stream_kernel<true>), dim3(stream_grid(true)), dim3(kStreamThreads), 0, s, nvec,
+                StreamSlot slot;
+                if (stream_slot_for(s, &slot, false)) {
+                    hipLaunchKernelGGL((adam_stream_kernel<true, true>), dim3(stream_grid(true)), dim3(kStreamThreads), 0, s, nvec,
+                                       ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
+                                       (f32x4 *)(v + head), h, slot.tickets, slot.done_word, slot.number);
+                    return false;
+                }
+                hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec);
+                hipLaunchKernelGGL((adam_stream_kernel<true, false>), dim3(stream_grid(true)), dim3(kStreamThreads), 0, s, nvec,
                                    ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
-                                   (f32x4 *)(v + head), h);
+                                   (f32x4 *)(v + head), h, (uint32_t *)nullptr, (uint32_t *)nullptr, 0u);
                 hipLaunchKernelGGL((adam_stream_finish_kernel<Half>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
                                    out16, nvec);
                 return false;
@@ -671,7 +699,7 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_multi_kernel(AdamB
         asm volatile("s_waitcnt vmcnt(4)" : "+v"(cur.g), "+v"(cur.p), "+v"(cur.m), "+v"(cur.v), "+v"(drawn));
         if (threadIdx.x == 0) handed[slot] = drawn;
         __syncthreads();
-        ahead = (int64_t)handed[slot] * kStreamCounters + which;
+        ahead = (int64_t)(handed[slot] + (gridDim.x >> 1)) * kStreamCounters + which;
         if (threadIdx.x == 0) stream_draw(drawn, counter);
         finish(cur, wcur);
         return tile;
@@ -769,8 +797,7 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
             }
         }
         if (counters_clear && groups >= (FP16 ? kStreamMinVecFp16 : kStreamMinVecBf16)) {
-            hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, (u32x2 *)batch.p16[batch.counter_tensor], most,
-                               stream_grid(FP16) / 2);
+            hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, (u32x2 *)batch.p16[batch.counter_tensor], most);
             hipLaunchKernelGGL((adam_stream_multi_kernel<FP16>), dim3(stream_grid(FP16)), dim3(kStreamThreads), 0, s,
                                batch, h);
             hipLaunchKernelGGL((adam_stream_multi_finish_kernel<FP16>), dim3(1), dim3(4 * kBatch + 64), 0, s, batch, h);

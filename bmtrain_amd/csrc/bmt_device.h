@@ -127,4 +127,25 @@ __device__ __forceinline__ void stream_draw(uint32_t &ticket, uint32_t *counter)
     asm volatile("global_atomic_add %0, %1, %2, off sc0" : "=v"(ticket) : "v"(counter), "v"(one) : "memory");
 }
 
+// ---- ticket counters that the library keeps for a stream (host side: stream_slot_for in bmt_host.h) ------------
+// A slot is a group of kSlotCounters counters, 4 KiB apart (counter c: word c * 1024 of the slot), plus a count of the
+// workgroups that have left the running launch (word 1).  The counters start at zero (the array is zero when the
+// library is loaded) and a launch leaves them at zero: every workgroup has received its last ticket before it leaves
+// (it waits for it), so when the last one leaves nothing is drawing any more; that workgroup puts the counters and
+// the count of leavers back to zero and then writes the launch's number into the slot's word of pinned host memory
+// (a release, so that the zeros are in memory first): from then on the host may hand the slot to another stream.
+constexpr int kSlotCounters = 8;
+__device__ __forceinline__ void stream_slot_leave(uint32_t *slot, uint32_t *done_word, uint32_t launch_number) {
+    if (threadIdx.x == 0) {
+        const uint32_t left = __hip_atomic_fetch_add(slot + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (left + 1 == gridDim.x) {
+#pragma unroll
+            for (int c = 0; c < kSlotCounters; c++)
+                __hip_atomic_store(slot + c * 1024, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(slot + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(done_word, launch_number, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+    }
+}
+
 }  // namespace bmt

@@ -654,7 +654,7 @@ __global__ __launch_bounds__(kFlatThreads) void ce_flat_vec_kernel(
 // on the per-thread default stream, or beyond the slot table keep the workgroup-per-tile kernel.
 constexpr int kFlatStreamThreads = 256;
 constexpr int kFlatStreamVecs = 4;                    // vectors per lane and tile
-constexpr int kFlatCounters = 8;
+constexpr int kFlatCounters = kSlotCounters;
 constexpr int kFlatSlots = 256;
 // Smallest array (in 16-byte vectors) that runs as the resident grid: 2^27 elements, 256 MiB.  Measured against one
 // workgroup per tile, launches back to back on rows of 16,384 bf16 elements (% of peak, resident / per tile):
@@ -665,24 +665,6 @@ constexpr int32_t kFlatStreamMinRow = kFlatStreamThreads * kFlatStreamVecs * 8;
 // counter c of slot s: word c * 1024 + s * 4 (the counters of one launch sit 4 KiB apart); word s * 4 + 1 counts the
 // workgroups of the running launch that have left
 static __device__ __align__(256) uint32_t flat_tickets[kFlatCounters * 1024];
-
-// Counters start at zero (the array is zero when the library is loaded) and a launch leaves them at zero: every
-// workgroup has received its last ticket before it leaves (it waits for it), so when the last one leaves nothing
-// is drawing any more; that workgroup puts the eight counters and the count of leavers back to zero and then
-// writes the launch's number into the slot's word of pinned host memory (a release, so that the zeros are in
-// memory first): from then on the host may hand the slot to another stream.  No launch in front is needed.
-__device__ __forceinline__ void flat_leave(uint32_t *tickets, uint32_t *done_word, uint32_t launch_number) {
-    if (threadIdx.x == 0) {
-        const uint32_t left = __hip_atomic_fetch_add(tickets + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (left + 1 == gridDim.x) {
-#pragma unroll
-            for (int c = 0; c < kFlatCounters; c++)
-                __hip_atomic_store(tickets + c * 1024, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(tickets + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(done_word, launch_number, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-        }
-    }
-}
 
 template <typename T, int OP>
 __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
@@ -706,7 +688,7 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
     const int64_t first = (int64_t)q * kFlatCounters + which;
     int64_t ahead = (int64_t)(q + (gridDim.x >> 3)) * kFlatCounters + which;
     const uint32_t drawn_base = 2u * (gridDim.x >> 3);      // the first two tiles of a workgroup follow from its number
-    if (first >= ntiles) { flat_leave(tickets, done_word, launch_number); return; }
+    if (first >= ntiles) { stream_slot_leave(tickets, done_word, launch_number); return; }
     uint32_t drawn = 0;
     if (threadIdx.x == 0) stream_draw(drawn, counter);
     const uint32_t row_vecs = (uint32_t)n >> 3;
@@ -769,7 +751,7 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
         if (stage(b, a, 1) >= ntiles) break;
     }
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
-    flat_leave(tickets, done_word, launch_number);
+    stream_slot_leave(tickets, done_word, launch_number);
 }
 
 template <typename T, int OP>
@@ -919,7 +901,7 @@ static int ce_forward(int32_t m, int32_t n, const void *input, const void *targe
 //
 // Every device keeps a table of up to kFlatSlots stream handles; a stream's slot is its group of eight counters.
 // Launches that use a slot are numbered, and the last workgroup of a launch writes that number into the slot's word
-// of a small pinned host array (flat_leave).  When the table is full, the least recently used slot whose word shows
+// of a small pinned host array (stream_slot_leave).  When the table is full, the least recently used slot whose word shows
 // its latest launch — so nothing can still be drawing from its counters, whether or not its stream still exists — is
 // given to the new stream.  The handles in the table are only ever compared, never passed to the runtime: a stream
 // may have been destroyed since.  A process that creates and destroys streams therefore keeps the resident kernel.
@@ -935,15 +917,13 @@ struct FlatDevice {
     uint64_t clock = 0;
 };
 static FlatDevice flat_devices[64];
-struct FlatLaunch { uint32_t *tickets; uint32_t *done_word; uint32_t number; };
-
-static bool flat_tickets_for(hipStream_t stream, FlatLaunch *launch) {
+bool stream_slot_for(hipStream_t stream, StreamSlot *launch, bool counted) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
     auto fallback = [&]() -> bool {
         (void)hipGetLastError();
         std::lock_guard<std::mutex> lock(flat_mutex);
-        flat_stats[dev].fallback++;
+        if (counted) flat_stats[dev].fallback++;
         return false;
     };
     if (stream == hipStreamPerThread) return fallback();
@@ -959,7 +939,7 @@ static bool flat_tickets_for(hipStream_t stream, FlatLaunch *launch) {
         if (hipGetSymbolAddress((void **)&base, HIP_SYMBOL(flat_tickets)) != hipSuccess ||
             hipHostMalloc(&done, kFlatSlots * sizeof(uint32_t), hipHostMallocDefault) != hipSuccess) {
             (void)hipGetLastError();
-            flat_stats[dev].fallback++;
+            if (counted) flat_stats[dev].fallback++;
             return false;
         }
         for (int k = 0; k < kFlatSlots; k++) ((uint32_t *)done)[k] = 0u;
@@ -983,7 +963,7 @@ static bool flat_tickets_for(hipStream_t stream, FlatLaunch *launch) {
                 tried_up_to = d.slots[oldest].last_use;
                 if (d.done[oldest] == d.slots[oldest].launches) slot = oldest;
             }
-            if (slot < 0) { flat_stats[dev].fallback++; return false; }
+            if (slot < 0) { if (counted) flat_stats[dev].fallback++; return false; }
             flat_stats[dev].evictions++;
             d.slots[slot].stream = stream;
         }
@@ -992,7 +972,7 @@ static bool flat_tickets_for(hipStream_t stream, FlatLaunch *launch) {
     launch->number = ++d.slots[slot].launches;
     launch->tickets = d.base + slot * 4;
     launch->done_word = (uint32_t *)d.done + slot;
-    flat_stats[dev].resident++;
+    if (counted) flat_stats[dev].resident++;
     return true;
 }
 
@@ -1012,8 +992,8 @@ static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void 
         if (tiles < 1) tiles = 1;
         if (tiles > 0x7FFFFFFF) return fail(-1, "cross_entropy launcher: tensor too large for one launch");
         if (n % 8 == 0 && head == 0 && n >= kFlatStreamMinRow && total_vec >= kFlatStreamMinVec && total_vec < ((int64_t)1 << 32)) {
-            FlatLaunch fl;
-            if (flat_tickets_for(s, &fl)) {
+            StreamSlot fl;
+            if (stream_slot_for(s, &fl, true)) {
                 uint32_t *tickets = fl.tickets;
                 const int cus = device_cu_count();
                 const unsigned grid = (unsigned)(cus >= 64 ? cus / 64 * 64 : 64);      // 8 XCDs x 8 counters

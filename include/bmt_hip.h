@@ -24,16 +24,19 @@
  *     stream handles (which stream uses which group of ticket counters below) behind one mutex, 1 KiB of pinned host memory, the
  *     looked-up addresses of the two device arrays, and the cached compute-unit count;
  *   - device side, two fixed arrays in the library's own code object, one copy per GPU: 32 KiB of
- *     ticket counters for the in-place cross-entropy kernels (eight counters per stream in the table)
+ *     ticket counters for the in-place cross-entropy kernels and the long single-tensor Adam launches
+ *     (eight counters per stream in the table; every launch leaves them at zero)
  *     and the 4 MiB of partial sums of grad_stats_noalloc_launcher;
- *   - in a caller's buffer, only for the duration of a launch: long Adam launches keep four tile
- *     counters in the 16-bit parameter output (see adam_fp16_launcher).
+ *   - in a caller's buffer, only for the duration of a launch: long Adam launches on a stream without a
+ *     table entry, and long multi-tensor launches, keep four tile counters in the 16-bit parameter
+ *     output (see adam_fp16_launcher).
  * Launches that use a table entry are numbered, and the last workgroup of each writes its number into a
  * word of pinned host memory (1 KiB per device, allocated at the first such launch).  When the table is
  * full, the least recently used entry whose latest launch has left is given to the new stream; if the
- * entries looked at are all busy the launch runs the kernel that needs no counters (same results, a few
- * per cent slower).  Stream handles in the table are only compared, never handed to the runtime.  Launches on a stream under
- * graph capture, on hipStreamPerThread or on a stream of another device always take that kernel.
+ * entries looked at are all busy the launch does without an entry: the cross-entropy kernels run their
+ * one-tile-per-workgroup form, Adam keeps its counters in param_16 (same results, a few per cent
+ * slower).  Stream handles in the table are only compared, never handed to the runtime.  Launches on a
+ * stream under graph capture, on hipStreamPerThread or on a stream of another device never get an entry.
  */
 #ifndef BMT_HIP_H
 #define BMT_HIP_H
@@ -67,10 +70,13 @@ BMT_API int has_nan_inf_bf16_launcher(int64_t n, const void *g_bf16, void *mid, 
  * One fused step over n elements.  fp16 flavour: g is the loss-scaled gradient and
  * the moments are kept multiplied by `scale` (m in fp16, v in fp32).
  * Writes param_fp32, param_fp16 (round-to-nearest-even), m_fp16, v_fp32.  n <= 0: no-op.
- * param_fp16 is output only and its previous contents are never read: while a launch of 2^24
- * elements or more (bf16 flavour: 12,582,912 or more) is in flight, four of its last 1,537 8-byte groups hold tile counters (set by a
- * small kernel in front, replaced by the real values by one behind, in stream order).  A call whose
- * param_fp16 overlaps g_fp16, param_fp32, m_fp16 or v_fp32 returns -1, at any size.
+ * param_fp16 is output only and its previous contents are never read.  A launch of 2^24 elements or
+ * more (bf16 flavour: 12,582,912 or more) hands out its tiles through counters: those of the
+ * stream's entry in the library's table (see "State" above) or, where the stream has none (graph
+ * capture, hipStreamPerThread, table busy), four of the last 1,537 8-byte groups of param_fp16,
+ * which then hold counters while the launch is in flight (set by a small kernel in front, replaced
+ * by the real values by one behind, in stream order).  A call whose param_fp16 overlaps g_fp16,
+ * param_fp32, m_fp16 or v_fp32 returns -1, at any size and on any stream.
  */
 BMT_API int adam_fp16_launcher(int64_t n, void *param_fp32, void *param_fp16, const void *g_fp16,
                        void *m_fp16, void *v_fp32,

@@ -307,10 +307,10 @@ def test_one_transformer_block_flat_buffer():
                                    ((3 << 22) + 1020, 4)])
 def test_around_the_launch_size_where_the_resident_grid_takes_over(flavour, n, off):
     """From 3 * 2^20 (bf16) or 2^22 (fp16) four-element groups on, a resident grid draws tiles of 256 groups from four
-    counters kept in the 16-bit output (word 0 of the vectors nvec-1, nvec-513, nvec-1025, nvec-1537), whose real
-    values a small kernel restores afterwards.  Whole-buffer comparison with the oracle just below and above both
-    sizes, with unaligned heads and partial last tiles: every tile stepped exactly once, and the counters' places
-    hold their real values.  A resident launch starts its tiles at the fp32 parameters' next 4 KiB boundary and leaves
+    counters: a slot of the library's own array when the stream has one (here), else places in the 16-bit output
+    (word 0 of the vectors nvec-1, nvec-513, nvec-1025, nvec-1537; covered under graph capture in
+    test_gpu_streams_graphs.py).  Whole-buffer comparison with the oracle just below and above both sizes, with
+    unaligned heads and partial last tiles: every tile stepped exactly once, every 16-bit value in place.  A resident launch starts its tiles at the fp32 parameters' next 4 KiB boundary and leaves
     the up to 1,023 elements in front of it to the element kernel (offsets 1 to 1,000 below), unless that would take
     the call below the size of a resident launch (the last two cases)."""
     dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16

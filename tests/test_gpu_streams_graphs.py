@@ -261,3 +261,95 @@ def test_host_threads_launching_at_once_on_their_own_streams():
         th.join(timeout=100)
     assert not any(th.is_alive() for th in threads)
     assert failures == []
+
+
+@pytest.mark.parametrize("flavour", ["bf16", "fp16"])
+def test_long_adam_launch_with_and_without_the_library_s_counters(flavour):
+    """A resident Adam launch draws its tiles from counters: a slot of the library's own array when the stream has
+    one, else (here: under graph capture) four places in the 16-bit output that a kernel in front zeroes and a kernel
+    behind overwrites with the real values.  Three steps each way on twin states, from views 5 elements into their
+    buffers: same bits after every step, and the first step equal to the oracle."""
+    n, off = (1 << 24) + 4 * 2048 + 3, 5
+    dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
+    mdt = torch.float16 if flavour == "fp16" else torch.float32
+    scale = 16.0 if flavour == "fp16" else 1.0
+    fn = OF.adam_fp16 if flavour == "fp16" else OF.adam_bf16
+    gen = torch.Generator().manual_seed(31)
+    host = [torch.randn(n, generator=gen) * 0.02, torch.zeros(n, dtype=dt16), (torch.randn(n, generator=gen) * 1e-3 * scale).to(dt16),
+            (torch.randn(n, generator=gen) * 1e-4 * scale).to(mdt), (torch.randn(n, generator=gen) * 1e-6 * scale).abs()]
+
+    def place():
+        views = []
+        for t in host:
+            buf = torch.full((n + 64,), -1, dtype=t.dtype, device="cuda")
+            buf[off:off + n] = t.cuda()
+            views.append(buf[off:off + n])
+        return views
+    eager, graphed = place(), place()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                         # warm-up outside capture, on a scratch copy
+        fn(*[t.clone() for t in graphed], 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, 1)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn(*graphed, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, 1)
+    for replay in range(3):
+        fn(*eager, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, 1)
+        graph.replay()
+        torch.cuda.synchronize()
+        for x, y in zip(eager, graphed):
+            assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), replay
+        if replay == 0:
+            p, v = host[0].numpy().copy(), host[4].numpy().copy()
+            h = np.zeros(n, np.uint16)
+            bc1, bc2 = oracle.bias_corrections(0.9, 0.999, 1)
+            if flavour == "fp16":
+                m = bits16(host[3])
+                oracle.adam_gpu_fp16(p, h, bits16(host[2]), m, v, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, bc1, bc2)
+                assert np.array_equal(bits16(graphed[3]), m)
+            else:
+                m = host[3].numpy().copy()
+                oracle.adam_gpu_bf16(p, h, bits16(host[2]), m, v, 0.9, 0.999, 1e-8, 1e-3, scale, 0.01, bc1, bc2)
+                assert np.array_equal(f32_bits(graphed[3].cpu().numpy()), f32_bits(m))
+            assert np.array_equal(f32_bits(graphed[0].cpu().numpy()), f32_bits(p))
+            assert np.array_equal(f32_bits(graphed[4].cpu().numpy()), f32_bits(v))
+            assert np.array_equal(bits16(graphed[1]), h)
+
+
+def test_long_adam_launches_on_more_streams_than_the_library_keeps_counters_for():
+    """264 runtime streams, each stepping a state of its own (same contents) by one resident-size launch, all in flight
+    together: the streams beyond the table's 256 entries get an entry whose launch has completed or fall back to the
+    counters in the 16-bit output; no two running launches may share counters — every state comes out like the first,
+    and the first like a launch made alone."""
+    hip, ctypes = _runtime()
+    n = (3 << 22) + 4 * 300 + 1
+    proto = _state(n, 41)
+    alone = [t.clone() for t in proto]
+    OF.adam_bf16(*alone, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 3)
+    torch.cuda.synchronize()
+    handles = []
+    try:
+        for _ in range(264):
+            handle = ctypes.c_void_p()
+            assert hip.hipStreamCreate(ctypes.byref(handle)) == 0
+            handles.append(handle)
+        states = [[proto[0].clone(), torch.zeros_like(proto[1]), proto[2], proto[3].clone(), proto[4].clone()] for _ in handles]
+        torch.cuda.synchronize()
+        for rnd in range(2):
+            for handle, st in zip(handles, states):
+                with torch.cuda.stream(torch.cuda.ExternalStream(handle.value)):
+                    OF.adam_bf16(*st, 0.9, 0.999, 1e-8, 1e-3, 1.0, 0.01, 3 + rnd)
+            torch.cuda.synchronize()
+            if rnd == 0:
+                for k, st in enumerate(states):
+                    for x, y in zip(st, alone):
+                        assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), k
+        for k, st in enumerate(states[1:]):
+            for x, y in zip(st, states[0]):
+                assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)), k
+    finally:
+        torch.cuda.synchronize()
+        for handle in handles:
+            hip.hipStreamDestroy(handle)
