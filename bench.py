@@ -242,7 +242,7 @@ def other_workloads(torch, dev, LF, OF, iters=20):
     sumsq = torch.zeros(1, dtype=torch.float64, device=dev)
     flag = torch.zeros(1, dtype=torch.uint8, device=dev)
     out["grad_stats_bf16_202M"] = entry(timed(lambda: OF.grad_stats(grad, sumsq, flag)), 2 * n)
-    # single mid-size tensors, as per-tensor stepping of a model meets them: below 12,582,912 elements a bf16 launch is
+    # single mid-size tensors, as per-tensor stepping of a model meets them: below 10,485,760 elements a bf16 launch is
     # one workgroup per tile, from there on the resident grid (launches back to back, so each figure holds one launch gap)
     for label, k in (("adam_bf16_one_tensor_2^22", 1 << 22), ("adam_bf16_one_tensor_2^23", 1 << 23),
                      ("adam_bf16_one_tensor_12.6M", 3 << 22), ("adam_bf16_one_tensor_4096x4096", 1 << 24),

@@ -238,12 +238,16 @@ constexpr int kStreamThreads = 256;
 constexpr int kStreamCounters = 4;
 constexpr int64_t kStreamCounterStride = 512;            // in 8-byte vectors: 4 KiB
 // Smallest launch (in 4-element groups) that runs as the resident grid, where it overtakes one workgroup per
-// tile.  Measured per flavour with the counters in the 16-bit output, launches back to back:
-//   bf16   10.5 M elements: 71 % of peak either way;  12.6 M: 74.3 against 71.7;  14.7 M: 76.2 against 73.9;
-//          8.4 M: 70.3 against 74.0;  4.2 M: 58.7 against 70.7
-//   fp16   12.6 M: 70.2 against 73.2;  16.8 M: 73.2 against 73.9;  202 M: 80.0 against 72.8
-constexpr int64_t kStreamMinVecBf16 = (int64_t)3 << 20;   // 12,582,912 elements
-constexpr int64_t kStreamMinVecFp16 = (int64_t)1 << 22;   // 16,777,216 elements
+// tile.  Measured per flavour, launches back to back, % of peak of one workgroup per tile / of the resident grid
+// with the stream's own counters (a single kernel):
+//   bf16    8.4 M elements 73.5 / 67.7;  10.5 M 73.6 / 74.4;  12.6 M 72.5 / 75.9;  16.8 M 73.5 / 78.7;  33.6 M 72.3 / 81.9
+//   fp16   16.8 M 75.1 / 72.7;  21.0 M 75.5 / 74.1;  25.2 M 74.3 / 75.0;  33.6 M 76.3 / 77.2;  45 M 74.6 / 76.4;  202 M 72.8 / 80
+// Multi-tensor batches keep their counters in a 16-bit output (three kernels) and change over a little later:
+//   bf16   10.5 M: 71 either way;  12.6 M: 71.7 / 74.3;  14.7 M: 73.9 / 76.2
+constexpr int64_t kStreamMinVecBf16 = (int64_t)5 << 19;        // 10,485,760 elements
+constexpr int64_t kStreamMinVecFp16 = (int64_t)3 << 21;        // 25,165,824 elements
+constexpr int64_t kStreamMultiMinVecBf16 = (int64_t)3 << 20;   // 12,582,912 elements
+constexpr int64_t kStreamMultiMinVecFp16 = (int64_t)3 << 21;   // 25,165,824 elements
 
 __device__ __forceinline__ bool holds_stream_counter(int64_t i, int64_t nvec) {
     const int64_t d = nvec - 1 - i;
@@ -769,7 +773,7 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
     auto flush = [&]() -> hipError_t {
         if (batch.count == 0) return hipSuccess;
         const uint32_t tiles = batch.first_tile[batch.count];
-        // Batches of kStreamMinVec* groups or more run as the resident grid; the tensor with the most groups (at
+        // Batches of kStreamMultiMinVec* groups or more run as the resident grid; the tensor with the most groups (at
         // least 3 * 2^20 / 32 of them, so the four counter places exist) lends its 16-bit output to the counters.
         int64_t groups = 0, most = -1;
         batch.stream_first[0] = 0;
@@ -796,7 +800,7 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
                                  !overlaps(lo, span * 8, batch.p16[c], 2 * nc);
             }
         }
-        if (counters_clear && groups >= (FP16 ? kStreamMinVecFp16 : kStreamMinVecBf16)) {
+        if (counters_clear && groups >= (FP16 ? kStreamMultiMinVecFp16 : kStreamMultiMinVecBf16)) {
             hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, (u32x2 *)batch.p16[batch.counter_tensor], most);
             hipLaunchKernelGGL((adam_stream_multi_kernel<FP16>), dim3(stream_grid(FP16)), dim3(kStreamThreads), 0, s,
                                batch, h);

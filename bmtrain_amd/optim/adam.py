@@ -41,7 +41,7 @@ class AdamOptimizer(torch.optim.Optimizer):
         super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
         self._hold_steps = hold_steps
         # Tensors share launches, up to 32 per launch (same arithmetic per element as one launch per tensor,
-        # which remains available by setting batch_launches to False); a batch of 12.6 M (bf16) or 2^24 (fp16) elements or more runs as
+        # which remains available by setting batch_launches to False); a batch of 12.6 M (bf16) or 25.2 M (fp16) elements or more runs as
         # one resident grid over all its tensors.  Tensors of `alone_from` elements or more are long launches
         # by themselves.
         self.batch_launches = True

@@ -70,8 +70,8 @@ BMT_API int has_nan_inf_bf16_launcher(int64_t n, const void *g_bf16, void *mid, 
  * One fused step over n elements.  fp16 flavour: g is the loss-scaled gradient and
  * the moments are kept multiplied by `scale` (m in fp16, v in fp32).
  * Writes param_fp32, param_fp16 (round-to-nearest-even), m_fp16, v_fp32.  n <= 0: no-op.
- * param_fp16 is output only and its previous contents are never read.  A launch of 2^24 elements or
- * more (bf16 flavour: 12,582,912 or more) hands out its tiles through counters: those of the
+ * param_fp16 is output only and its previous contents are never read.  A launch of 25,165,824 elements
+ * or more (bf16 flavour: 10,485,760 or more) hands out its tiles through counters: those of the
  * stream's entry in the library's table (see "State" above) or, where the stream has none (graph
  * capture, hipStreamPerThread, table busy), four of the last 1,537 8-byte groups of param_fp16,
  * which then hold counters while the launch is in flight (set by a small kernel in front, replaced
@@ -175,7 +175,7 @@ BMT_API int fused_softmax_inplace_bf16_launcher(int32_t m, int32_t n, void *logi
  * `count` tensors that share their hyper-parameters (same group, same step count) in as few launches as
  * possible; per element the arithmetic is that of adam_{fp16,bf16}_launcher, bit for bit.
  * `tensors` is a host array; `m` is float[n] for bf16 and half[n] for fp16.  Entries with n <= 0 are skipped.
- * param_16 is output only; a launch over 2^24 elements or more (bf16: 12,582,912 or more) keeps four tile counters in the
+ * param_16 is output only; a launch over 25,165,824 elements or more (bf16: 12,582,912 or more) keeps four tile counters in the
  * param_16 of its largest tensor while it runs (as adam_fp16_launcher does).  The whole table is checked before
  * the first launch: the call returns -1, and no tensor has been stepped, if any entry has a null pointer or a
  * param_16 that overlaps an input of the same tensor.  A batch in which another entry shares memory with the

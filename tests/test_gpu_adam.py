@@ -304,9 +304,10 @@ def test_one_transformer_block_flat_buffer():
                                    ((1 << 24) - 1, 0), ((1 << 24) + 2, 2), ((1 << 24) + 1024 * 7 + 5, 1), ((1 << 24) + 4 * 2048 + 3, 0),
                                    ((1 << 25) + 12345, 0), ((1 << 25) + 4096 * 3 + 1, 2), (3 * (1 << 24) + 4 * 1537, 3),
                                    ((1 << 24) + 77, 8), ((3 << 22) + 5000, 256), ((1 << 25) + 1, 1000), ((3 << 22) + 1023, 1),
-                                   ((3 << 22) + 1020, 4)])
+                                   ((3 << 22) + 1020, 4), ((5 << 21) - 1, 0), ((5 << 21) + 2, 2), ((5 << 21) + 1023, 1),
+                                   ((3 << 23) - 1, 0), ((3 << 23) + 1024 * 7 + 5, 1), ((3 << 23) + 1020, 4)])
 def test_around_the_launch_size_where_the_resident_grid_takes_over(flavour, n, off):
-    """From 3 * 2^20 (bf16) or 2^22 (fp16) four-element groups on, a resident grid draws tiles of 256 groups from four
+    """From 10,485,760 (bf16) or 25,165,824 (fp16) elements on, a resident grid draws tiles of 256 groups from four
     counters: a slot of the library's own array when the stream has one (here), else places in the 16-bit output
     (word 0 of the vectors nvec-1, nvec-513, nvec-1025, nvec-1537; covered under graph capture in
     test_gpu_streams_graphs.py).  Whole-buffer comparison with the oracle just below and above both sizes, with
@@ -421,7 +422,7 @@ def test_multi_tensor_launch_equals_per_tensor_launches(flavour):
 
 @pytest.mark.parametrize("flavour", ["bf16", "fp16"])
 def test_long_multi_tensor_launch_runs_as_one_resident_grid(flavour):
-    """Batches of 3 * 2^22 (bf16) or 2^24 (fp16) elements or more run as one resident grid over all their tensors: tiles of 256 groups numbered
+    """Batches of 3 * 2^22 (bf16) or 3 * 2^23 (fp16) elements or more run as one resident grid over all their tensors: tiles of 256 groups numbered
     through the tensors, drawn by ticket from four counters kept in the 16-bit output of the largest tensor; leftover
     elements and the counters' places are finished by a small kernel.  40 tensors (two launches, the second a short
     one), 33 equal tensors, and a mix of sizes from 3 to 2^24 + 5 elements with every leftover count — bit for bit
@@ -432,7 +433,8 @@ def test_long_multi_tensor_launch_runs_as_one_resident_grid(flavour):
     for sizes in ([1_200_001 + 4 * k for k in range(39)] + [2_000_003], [1_200_000] * 32 + [4096 * 300 + 3],
                   [(1 << 24) + 5, 77, 4096, (1 << 22) + 2, 3, 1_000_001, 255, 1024, 1023, 6, (1 << 23) + 3],
                   [(1 << 22) + 1, (1 << 23) + 2, 4099, 255],          # 12.6 M elements: resident for bf16, short kernel for fp16
-                  [(3 << 22) - 8192, 4096, 4097]):                     # just above the bf16 size, the largest tensor just below it
+                  [(3 << 22) - 8192, 4096, 4097],                      # just above the bf16 size, the largest tensor just below it
+                  [(3 << 23) - 8192, 4096, 4097]):                     # the same at the fp16 size
         gen = torch.Generator(device="cuda").manual_seed(len(sizes))
         single, multi = [], []
         for n in sizes:

@@ -269,7 +269,7 @@ def test_long_adam_launch_with_and_without_the_library_s_counters(flavour):
     one, else (here: under graph capture) four places in the 16-bit output that a kernel in front zeroes and a kernel
     behind overwrites with the real values.  Three steps each way on twin states, from views 5 elements into their
     buffers: same bits after every step, and the first step equal to the oracle."""
-    n, off = (1 << 24) + 4 * 2048 + 3, 5
+    n, off = (1 << 25) + 4 * 2048 + 3, 5                  # resident size for both flavours
     dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
     mdt = torch.float16 if flavour == "fp16" else torch.float32
     scale = 16.0 if flavour == "fp16" else 1.0
