@@ -448,6 +448,33 @@ def full_model_side_measurements(torch, OF, p16, grad, p32, mom, var, iters=5):
                                     "frac": round(2 * n / (mean * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
     layer = [(4096, 4096)] * 4 + [(11008, 4096)] * 2 + [(4096, 11008)] + [(4096,)] * 2
     shapes = [(32000, 4096)] + layer * 32 + [(4096,), (32000, 4096)]
+    # the same gradients as the 291 tensors of the model, handed over as a list (as separately allocated
+    # gradients are): one launch per 64 tensors against one or two launches per tensor
+    from bmtrain_amd.loss import _function as LF
+    pieces, lo = [], 0
+    for shape in shapes:
+        size = 1
+        for d in shape:
+            size *= d
+        pieces.append(grad[lo:lo + size])
+        lo += size
+
+    def per_tensor(with_sum):
+        for g in pieces:
+            if with_sum:
+                OF.grad_stats(g, sumsq, flag)
+            else:
+                LF.has_inf_nan(g, flag)
+    for label, fn in (("has_inf_nan_291_tensors_multi_launch", lambda: OF.grad_stats_multi(pieces, None, flag)),
+                      ("has_inf_nan_291_tensors_launch_per_tensor", lambda: per_tensor(False)),
+                      ("grad_stats_291_tensors_multi_launch", lambda: OF.grad_stats_multi(pieces, sumsq, flag)),
+                      ("grad_stats_291_tensors_launch_per_tensor", lambda: per_tensor(True))):
+        fn()
+        torch.cuda.synchronize()
+        mean, median, low = timed_batches(torch, fn, 8, 1)
+        out[label] = {"ms": round(mean, 4), "ms_median": round(median, 4), "ms_min": round(low, 4),
+                      "achieved_GBps": round(2 * n / (mean * 1e-3) / 1e9, 1),
+                      "frac": round(2 * n / (mean * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
     gen = torch.Generator(device=grad.device).manual_seed(44)
     for label, defer in (("eager", False), ("deferred", True)):
         params, lo = [], 0

@@ -129,12 +129,29 @@ def _bind_multi(name, extra_floats=0):
     return call
 
 
+class ScanTensor(ctypes.Structure):
+    """`bmt_scan_tensor` of include/bmt_hip.h."""
+    _fields_ = [("g_16", _p), ("n", _i64)]
+
+
+_lib.grad_stats_multi_launcher.argtypes = [_i32, ctypes.POINTER(ScanTensor), _i32, _p, _p, _p, _p]
+_lib.grad_stats_multi_launcher.restype = ctypes.c_int
+
+
+def grad_stats_multi_launcher(tensors, is_bf16, sumsq, flag, workspace, stream):
+    """tensors: sequence of (grad_16_ptr, n); sumsq / workspace may be 0 (flag only)."""
+    table = (ScanTensor * len(tensors))(*[ScanTensor(*t) for t in tensors])
+    status = _lib.grad_stats_multi_launcher(len(tensors), table, is_bf16, sumsq, flag, workspace, stream)
+    if status != 0:
+        raise RuntimeError(f"grad_stats_multi_launcher failed with status {status}: {last_error()}")
+
+
 adam_bf16_multi_launcher = _bind_multi("adam_bf16_multi_launcher")
 adam_fp16_multi_launcher = _bind_multi("adam_fp16_multi_launcher")
 adam_bf16_multi_clip_launcher = _bind_multi("adam_bf16_multi_clip_launcher", 1)
 adam_fp16_multi_clip_launcher = _bind_multi("adam_fp16_multi_clip_launcher", 1)
 
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["is_bf16_supported", "bmt_hip_last_error", "grad_stats_workspace_floats",
-                                                  "bmt_hip_flat_stream_stats",
+                                                  "bmt_hip_flat_stream_stats", "grad_stats_multi_launcher",
                                                   "adam_bf16_multi_launcher", "adam_fp16_multi_launcher",
                                                   "adam_bf16_multi_clip_launcher", "adam_fp16_multi_clip_launcher"])

@@ -225,6 +225,157 @@ static float *static_partials(hipStream_t stream, const char **why) {
     return ptr;
 }
 
+// ---- the same two passes over several gradient tensors at once ------------------------------------
+// A model whose gradients are separate allocations is scanned tensor by tensor otherwise: the 291 tensors of a
+// 6.74 B-parameter model cost 2.35 ms (flag) / 3.46 ms (flag and sum of squares, two launches each) against
+// 1.8 / 1.9 ms for one flat buffer, all of the difference launches; here 1.92 / 1.96 ms.  Up to kScanBatch tensors
+// travel in the kernel arguments; tiles are numbered through the tensors, a workgroup finds its tensor from the
+// table in the arguments, and the first tile of a tensor also takes that tensor's elements in front of and behind
+// its 16-byte vectors.  The partial sums are one per tile, as in the single-tensor kernel.
+constexpr int kScanBatch = 64;
+// Vectors per lane of the flag-only pass: the search in front makes a workgroup's start longer than the
+// single-tensor kernel's, and two vectors spread it (1 / 2 / 4 / 8 vectors: 65 / 87 / 81 / 86 % of the HBM
+// peak over the 291 gradient tensors of a 6.74 B-parameter model).
+constexpr int kScanMultiUnroll = 2;
+// first_tile[k]: number of the first tile of tensor k; first_tile[count] = tiles of the launch; entries behind it
+// hold 0xFFFFFFFF.  Every tensor has at least one tile, so the used entries rise strictly.  every_4th[j] repeats
+// first_tile[4 j]: a workgroup finds its tensor with two rounds of scalar loads (16 entries, then the 4 between
+// two of them) instead of the six dependent ones of a bisection - the search runs in front of the workgroup's
+// only loads of data, so every round of it is time the memory pipeline of that workgroup's slot stands idle.
+struct ScanBatch {
+    const uint16_t *g[kScanBatch];
+    int64_t n[kScanBatch];
+    uint32_t first_tile[kScanBatch + 4];
+    uint32_t every_4th[kScanBatch / 4];
+    int32_t count;
+};
+
+template <typename T, bool STATS>
+__global__ __launch_bounds__(kScanThreads) void scan_multi_kernel(ScanBatch batch, uint8_t *__restrict__ flag,
+                                                                   float *__restrict__ partials) {
+    constexpr int UNROLL = STATS ? kStatsUnroll : kScanMultiUnroll;
+    int group = -1;                                    // every_4th[group] <= blockIdx.x < every_4th[group + 1]
+#pragma unroll
+    for (int j = 0; j < kScanBatch / 4; j++) group += batch.every_4th[j] <= blockIdx.x ? 1 : 0;
+    const uint32_t *four = batch.first_tile + 4 * group;
+    const uint32_t f0 = four[0], f1 = four[1], f2 = four[2], f3 = four[3];
+    const int within = (f1 <= blockIdx.x ? 1 : 0) + (f2 <= blockIdx.x ? 1 : 0) + (f3 <= blockIdx.x ? 1 : 0);
+    const int lo = 4 * group + within;
+    const uint32_t first = within == 0 ? f0 : within == 1 ? f1 : within == 2 ? f2 : f3;
+    const uint16_t *g = batch.g[lo];
+    const int64_t n = batch.n[lo];
+    const uint32_t tile = blockIdx.x - first;
+    int64_t head = (int64_t)(((16 - ((uintptr_t)g & 15u)) & 15u) / 2);
+    if (head > n) head = n;
+    const int64_t nvec = (n - head) / 8;
+    const u32x4 *body = (const u32x4 *)(g + head);
+    const int64_t base = (int64_t)tile * (kScanThreads * UNROLL) + threadIdx.x;
+    uint32_t hit = 0;
+    float acc = 0.f;
+    u32x4 w[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const int64_t i = base + (int64_t)u * kScanThreads;
+        if (i < nvec) w[u] = __builtin_nontemporal_load(body + i);
+        else w[u] = u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            hit |= exp_all_ones2<T>(w[u][k]);
+            if (STATS) acc = sumsq2<T>(w[u][k], acc);
+        }
+    }
+    if (tile == 0) {   // unaligned head and tail of this tensor, one element per lane
+        const int64_t tail_lo = head + nvec * 8;
+        const int64_t edge = head + (n - tail_lo);
+        if ((int64_t)threadIdx.x < edge) {
+            const int64_t i = (int64_t)threadIdx.x < head ? (int64_t)threadIdx.x : tail_lo + ((int64_t)threadIdx.x - head);
+            hit |= exp_all_ones2<T>((uint32_t)g[i]);
+            if (STATS) {
+                const float x = T::to_f32(g[i]);
+                acc = __builtin_fmaf(x, x, acc);
+            }
+        }
+    }
+    if (!STATS) {
+        if (__builtin_amdgcn_ballot_w64(hit != 0) != 0 && (threadIdx.x & (kWave - 1)) == 0 &&
+            __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+            __hip_atomic_store(flag, (uint8_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    __shared__ float slots[kScanThreads / kWave];
+    __shared__ uint32_t any_wave;
+    if (threadIdx.x == 0) any_wave = 0;
+    __syncthreads();
+    if (__builtin_amdgcn_ballot_w64(hit != 0) != 0 && (threadIdx.x & (kWave - 1)) == 0) any_wave = 1;
+    const float total = block_allreduce<false>(acc, slots);   // contains a barrier
+    if (threadIdx.x == 0) {
+        partials[blockIdx.x] = total;
+        if (any_wave) __hip_atomic_store(flag, (uint8_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+template <typename T>
+static int scan_multi(int32_t count, const bmt_scan_tensor *tensors, void *sumsq, void *flag, void *workspace, void *stream,
+                      const char *who) {
+    if (count <= 0) return 0;
+    if (!tensors) return fail(-1, "grad_stats_multi_launcher: null tensor table");
+    if (!flag) return fail(-1, "grad_stats_multi_launcher: null flag");
+    if (sumsq && !workspace) return fail(-1, "grad_stats_multi_launcher: sumsq without workspace");
+    if ((uintptr_t)sumsq & 7u) return fail(-1, "grad_stats_multi_launcher: sumsq must be 8-byte aligned");
+    const int64_t per_tile = (int64_t)kScanThreads * (sumsq ? kStatsUnroll : kScanMultiUnroll) * 8;     // elements
+    for (int32_t k = 0; k < count; k++) {              // the whole table first: an error means nothing was launched
+        if (tensors[k].n <= 0) continue;
+        if (!tensors[k].g_16) return fail(-1, "grad_stats_multi_launcher: null pointer");
+        if ((uintptr_t)tensors[k].g_16 & 1u) return fail(-1, "grad_stats_multi_launcher: gradient pointer is not 2-byte aligned");
+        if (tensors[k].n / per_tile + 1 > 0x3FFFFFFF) return fail(-1, "grad_stats_multi_launcher: tensor too large for one launch");
+    }
+    ScanBatch batch;
+    batch.count = 0;
+    batch.first_tile[0] = 0;
+    auto flush = [&]() -> hipError_t {
+        if (batch.count == 0) return hipSuccess;
+        const uint32_t tiles = batch.first_tile[batch.count];
+        for (int k = batch.count + 1; k < kScanBatch + 4; k++) batch.first_tile[k] = 0xFFFFFFFFu;
+        for (int j = 0; j < kScanBatch / 4; j++) batch.every_4th[j] = batch.first_tile[4 * j];
+        if (sumsq) {
+            hipLaunchKernelGGL((scan_multi_kernel<T, true>), dim3(tiles), dim3(kScanThreads), 0, (hipStream_t)stream, batch,
+                               (uint8_t *)flag, (float *)workspace);
+            hipLaunchKernelGGL(grad_stats_finish_kernel, dim3(1), dim3(kScanThreads), 0, (hipStream_t)stream,
+                               (const float *)workspace, (int64_t)tiles, (double *)sumsq);
+        } else {
+            hipLaunchKernelGGL((scan_multi_kernel<T, false>), dim3(tiles), dim3(kScanThreads), 0, (hipStream_t)stream, batch,
+                               (uint8_t *)flag, (float *)nullptr);
+        }
+        batch.count = 0;
+        batch.first_tile[0] = 0;
+        return hipGetLastError();
+    };
+    for (int32_t k = 0; k < count; k++) {
+        const int64_t n = tensors[k].n;
+        if (n <= 0) continue;
+        const uintptr_t a = (uintptr_t)tensors[k].g_16;
+        int64_t head = (int64_t)(((16 - (a & 15u)) & 15u) / 2);
+        if (head > n) head = n;
+        const int64_t nvec = (n - head) / 8;
+        int64_t tiles = (nvec * 8 + per_tile - 1) / per_tile;
+        if (tiles < 1) tiles = 1;
+        if (batch.count == kScanBatch || (int64_t)batch.first_tile[batch.count] + tiles > 0x7FFFFFFF) {
+            hipError_t e = flush();
+            if (e != hipSuccess) return fail((int)e, who, e);
+        }
+        const int c = batch.count;
+        batch.g[c] = (const uint16_t *)tensors[k].g_16;
+        batch.n[c] = n;
+        batch.first_tile[c + 1] = batch.first_tile[c] + (uint32_t)tiles;
+        batch.count = c + 1;
+    }
+    hipError_t e = flush();
+    return e == hipSuccess ? 0 : fail((int)e, who, e);
+}
+
 }  // namespace bmt
 
 extern "C" int grad_stats_noalloc_launcher(int64_t n, const void *g_16, int32_t is_bf16, void *sumsq, void *flag, void *stream) {
@@ -260,4 +411,10 @@ extern "C" int grad_stats_fp16_launcher(int64_t n, const void *g_fp16, void *sum
 extern "C" int grad_stats_bf16_launcher(int64_t n, const void *g_bf16, void *sumsq, void *flag, void *workspace,
                                         void *stream) {
     return bmt::grad_stats<bmt::BFloat16>(n, g_bf16, sumsq, flag, workspace, stream, "grad_stats_bf16_launcher");
+}
+
+extern "C" int grad_stats_multi_launcher(int32_t count, const bmt_scan_tensor *tensors, int32_t is_bf16, void *sumsq, void *flag,
+                                         void *workspace, void *stream) {
+    return is_bf16 ? bmt::scan_multi<bmt::BFloat16>(count, tensors, sumsq, flag, workspace, stream, "grad_stats_multi_launcher")
+                   : bmt::scan_multi<bmt::Half>(count, tensors, sumsq, flag, workspace, stream, "grad_stats_multi_launcher");
 }

@@ -141,6 +141,33 @@ def grad_stats(g_half: torch.Tensor, sumsq: torch.Tensor, flag: torch.Tensor) ->
     launcher(n, g_half.data_ptr(), sumsq.data_ptr(), flag.data_ptr(), workspace.data_ptr(), _current_stream())
 
 
+def grad_stats_multi(grads, sumsq, flag: torch.Tensor) -> None:
+    """``grad_stats`` (``sumsq`` a float64 tensor) or the overflow scan alone (``sumsq`` None) over a list of
+    16-bit gradients of one dtype, in one launch per 64 tensors instead of one or two per tensor — what a model
+    whose gradients are separate allocations needs (the loops of optim_manager.py:9-21 and :186-190)."""
+    if not grads:
+        return
+    dtype = grads[0].dtype
+    if dtype == torch.bfloat16:
+        _require_bf16()
+    elif dtype != torch.float16:
+        raise ValueError(f"grad_stats not supported for dtype {dtype}")
+    assert flag.is_cuda and flag.dtype == torch.uint8 and flag.numel() == 1, "flag must be one uint8 on cuda"
+    rows = []
+    for g in grads:
+        assert g.is_contiguous() and g.is_cuda, "gradients must be contiguous and on cuda"
+        assert g.dtype == dtype, "all gradients must share one 16-bit dtype"
+        rows.append((g.data_ptr(), g.numel()))
+    if sumsq is None:
+        C.grad_stats_multi_launcher(rows, int(dtype == torch.bfloat16), 0, flag.data_ptr(), 0, _current_stream())
+        return
+    assert sumsq.is_cuda and sumsq.dtype == torch.float64 and sumsq.numel() == 1, "sumsq must be one float64 on cuda"
+    floats = sum(C.grad_stats_workspace_floats(n) for _, n in rows)
+    workspace = torch.empty(floats, dtype=torch.float32, device=flag.device)
+    C.grad_stats_multi_launcher(rows, int(dtype == torch.bfloat16), sumsq.data_ptr(), flag.data_ptr(), workspace.data_ptr(),
+                                _current_stream())
+
+
 def adam_multi(tensors, beta1: float, beta2: float, eps: float, lr: float, scale: float, weight_decay: float,
                step: int, grad_coef: float = 1.0) -> None:
     """Fused GPU step over several parameter tensors that share hyper-parameters and step count.

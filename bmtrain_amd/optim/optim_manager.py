@@ -12,12 +12,29 @@ import torch
 from ..global_var import config
 from ..loss._function import has_inf_nan
 from ._base import flat_runs
-from ._function import grad_stats
+from ._function import grad_stats, grad_stats_multi
 
 
 def _scanned_grads(param_groups):
     """The gradients the overflow check looks at: those of non-fp32 parameters."""
     return [p.grad for group in param_groups for p in group["params"] if p.grad is not None and p.dtype != torch.float]
+
+
+def _scan(grads, sumsq, flag):
+    """The overflow scan (``sumsq`` None) or the scan with the sum of squares over 16-bit gradients: gradients that lie
+    back to back are read as one run, and several runs of one dtype share a launch."""
+    by_dtype = {}
+    for g in flat_runs(grads):
+        by_dtype.setdefault(g.dtype, []).append(g)
+    for dtype, runs in by_dtype.items():
+        if len(runs) > 1 and dtype in (torch.float16, torch.bfloat16):
+            grad_stats_multi(runs, sumsq, flag)
+        else:
+            for g in runs:
+                if sumsq is None:
+                    has_inf_nan(g, flag)
+                else:
+                    grad_stats(g, sumsq, flag)
 
 
 def _fingerprint(g):
@@ -34,8 +51,7 @@ def check_overflow(param_groups, known=None):
         flag = known[0]
     else:
         flag = torch.zeros(1, dtype=torch.uint8, device="cuda")[0]
-        for g in flat_runs(grads):      # gradients that lie back to back are scanned by one launch
-            has_inf_nan(g, flag)
+        _scan(grads, None, flag)
     if flag > 0:
         raise OverflowError("Gradient overflow")
 
@@ -221,8 +237,7 @@ class OptimManager:
                 # 16-bit gradients: one read of each tensor instead of an fp32 copy plus a norm
                 sumsq = torch.zeros(1, dtype=torch.float64, device=device)
                 flag = torch.zeros(1, dtype=torch.uint8, device=device)
-                for g in flat_runs(fused):
-                    grad_stats(g, sumsq, flag)
+                _scan(fused, sumsq, flag)
                 acc += sumsq.float()
                 scanned = (flag, [p.grad for p, g in zip(with_grad, grads) if id(g) in fused_ids])
             for g in grads:

@@ -239,6 +239,22 @@ BMT_API int grad_stats_noalloc_launcher(int64_t n, const void *g_16, int32_t is_
                                         void *stream);
 
 /*
+ * grad_stats_multi_launcher — no counterpart in the reference, whose overflow check and gradient norm loop
+ * over the parameters (bmtrain/optim/optim_manager.py:9-21, :186-190).  The passes of has_nan_inf_*_launcher
+ * (sumsq == NULL: only the sticky flag) or of grad_stats_*_launcher (sumsq != NULL: flag, and the sum of squares
+ * of all tensors accumulated into sumsq[0]) over `count` gradient tensors of one 16-bit type in as few launches
+ * as possible (64 tensors each).  `tensors` is a host array; entries with n <= 0 are skipped; the tensors may
+ * start at any 2-byte aligned address.  `workspace` (device, floats): at least the sum over the tensors of
+ * grad_stats_workspace_floats(n); not used when sumsq is NULL.  The table is checked before the first launch.
+ */
+typedef struct bmt_scan_tensor {
+    const void *g_16;
+    int64_t n;
+} bmt_scan_tensor;
+BMT_API int grad_stats_multi_launcher(int32_t count, const bmt_scan_tensor *tensors, int32_t is_bf16, void *sumsq,
+                                      void *flag, void *workspace, void *stream);
+
+/*
  * bmt_hip_flat_stream_stats — diagnostics, no counterpart in the reference.  For the current device, since the
  * library was loaded: out[0] = launches of the in-place cross-entropy / softmax kernels that ran as the resident
  * ticket-ordered grid, out[1] = large launches that could not get ticket counters (stream under capture,

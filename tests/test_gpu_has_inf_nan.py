@@ -208,3 +208,56 @@ def test_clip_grad_norm_uses_one_pass_and_matches_torch():
     coef = 64.0 / (want * 64 + 1e-6)
     for p, b in zip(ps, before):
         torch.testing.assert_close(p.grad.float(), (b.float() * coef).to(p.dtype).float(), rtol=2e-2, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_several_tensors_in_one_launch(dtype):
+    """grad_stats_multi_launcher: the overflow scan and the scan with the sum of squares over 150 tensors of 1 to
+    1.3 M elements at every 2-byte alignment (three launches of up to 64 tensors).  The flag equals the tensor-by-tensor
+    scan for a clean set and for an inf / NaN planted in turn in the first element, the last element, the unaligned
+    head and tail and the middle of several tensors; the sum of squares equals float64 arithmetic to 1e-6 and is the
+    same bits run after run."""
+    from bmtrain_amd.optim import _function as OF
+    from bmtrain_amd.loss import _function as LF
+    rnd = np.random.default_rng(5)
+    sizes = [1, 2, 7, 8, 9, 15, 16, 17, 1023, 8192, 8193, 65536 + 3] + [int(x) for x in rnd.integers(1, 1_300_000, 138)]
+    pool = torch.empty(sum(sizes) + 16 * len(sizes), dtype=dtype, device="cuda").normal_(0, 2.0)
+    grads, at = [], 0
+    for k, n in enumerate(sizes):
+        at += k % 8                                   # every 2-byte phase of a 16-byte vector
+        grads.append(pool[at:at + n])
+        at += n + (8 - at % 8) % 8 + 8
+    flag = torch.zeros(1, dtype=torch.uint8, device="cuda")
+    OF.grad_stats_multi(grads, None, flag)
+    assert flag.item() == 0
+    sums = []
+    for _ in range(2):
+        sumsq = torch.zeros(1, dtype=torch.float64, device="cuda")
+        OF.grad_stats_multi(grads, sumsq, flag)
+        sums.append(sumsq.view(torch.int64).item())
+        assert flag.item() == 0
+    assert sums[0] == sums[1]
+    exact = sum(g.double().pow(2).sum().item() for g in grads)
+    assert abs(torch.tensor(sums[0]).view(torch.float64).item() - exact) <= 1e-6 * exact
+    for k, where in ((0, 0), (3, -1), (11, 2), (11, -3), (40, 5), (70, -1), (149, 0), (100, None)):
+        g = grads[k]
+        i = g.numel() // 2 if where is None else (where if where >= 0 else g.numel() + where)
+        i = min(max(i, 0), g.numel() - 1)
+        keep = g[i].item()
+        for bad in (float("inf"), float("nan")):
+            g[i] = bad
+            for with_sum in (False, True):
+                flag.zero_()
+                OF.grad_stats_multi(grads, torch.zeros(1, dtype=torch.float64, device="cuda") if with_sum else None, flag)
+                single = torch.zeros(1, dtype=torch.uint8, device="cuda")
+                for t in grads:
+                    LF.has_inf_nan(t, single)
+                assert flag.item() == single.item() == 1, (k, i, bad, with_sum)
+        g[i] = keep
+    flag.zero_()
+    OF.grad_stats_multi(grads, None, flag)
+    assert flag.item() == 0
+    # nothing is launched for a table with a bad entry
+    from bmtrain_amd import C
+    with pytest.raises(RuntimeError, match="null pointer"):
+        C.grad_stats_multi_launcher([(grads[0].data_ptr(), 8), (0, 8)], 1, 0, flag.data_ptr(), 0, 0)

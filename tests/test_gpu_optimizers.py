@@ -275,8 +275,14 @@ def test_step_reuses_the_overflow_verdict_of_the_clipping_pass(monkeypatch):
     step() does not scan gradients nobody has written to since, and does scan again after an in-place write."""
     import bmtrain_amd.optim.optim_manager as om
     calls = []
-    real = om.has_inf_nan
+    real, real_multi = om.has_inf_nan, om.grad_stats_multi
     monkeypatch.setattr(om, "has_inf_nan", lambda g, flag: (calls.append(g.numel()), real(g, flag))[1])
+
+    def counted_multi(grads, sumsq, flag):          # several separate gradients share one launch
+        if sumsq is None:
+            calls.extend(g.numel() for g in grads)
+        return real_multi(grads, sumsq, flag)
+    monkeypatch.setattr(om, "grad_stats_multi", counted_multi)
     torch.manual_seed(8)
     ps = [torch.nn.Parameter(torch.randn(s, device="cuda").bfloat16()) for s in (5000, 77, 4096)]
     opt = bmt.optim.AdamOptimizer(ps, lr=1e-3)
