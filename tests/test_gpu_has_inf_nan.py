@@ -138,6 +138,40 @@ def test_full_size_buffers(name, dtype, n):
     # a strided sample agrees with the oracle
     sample = x[:: max(1, n // (1 << 20))].contiguous()
     assert gpu_flag(sample) == oracle_flag(sample, name)
+    if name == "bf16":
+        # the same buffer handed over as the 291 gradient tensors of the model (five launches of up to 64 tensors):
+        # the flag follows an inf / NaN at the seeded offsets, in a 4,096-element tensor and in the last element; the sum
+        # of squares equals the single-buffer pass to 1e-8 (the tiles, and so the fp32 partial sums, start elsewhere)
+        from bmtrain_amd.optim import _function as OF
+        x[n - 1] = keep_last = 0.0
+        layer = [4096 * 4096] * 4 + [11008 * 4096] * 3 + [4096] * 2
+        sizes = [32000 * 4096] + layer * 32 + [4096, 32000 * 4096]
+        assert sum(sizes) == n
+        pieces, lo = [], 0
+        for size in sizes:
+            pieces.append(x[lo:lo + size])
+            lo += size
+        flag = torch.zeros(1, dtype=torch.uint8, device="cuda")
+        whole, listed = torch.zeros(1, dtype=torch.float64, device="cuda"), torch.zeros(1, dtype=torch.float64, device="cuda")
+        OF.grad_stats(x, whole, flag)
+        OF.grad_stats_multi(pieces, listed, flag)
+        OF.grad_stats_multi(pieces, None, flag)
+        assert flag.item() == 0
+        assert abs(whole.item() - listed.item()) <= 1e-8 * whole.item() and whole.item() > 0
+        small = next(k for k, size in enumerate(sizes) if size == 4096)
+        for piece, at in ((None, a), (None, b), (pieces[small], 4095), (pieces[-1], sizes[-1] - 1), (pieces[0], 0)):
+            target = x if piece is None else piece
+            keep = target[at].clone()
+            for bad in (float("inf"), float("nan")):
+                target[at] = bad
+                for with_sum in (False, True):
+                    flag.zero_()
+                    OF.grad_stats_multi(pieces, torch.zeros(1, dtype=torch.float64, device="cuda") if with_sum else None, flag)
+                    assert flag.item() == 1, (at, bad, with_sum)
+            target[at] = keep
+        flag.zero_()
+        OF.grad_stats_multi(pieces, None, flag)
+        assert flag.item() == 0
     del x
     torch.cuda.empty_cache()
 
