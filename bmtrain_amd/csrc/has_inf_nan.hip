@@ -228,26 +228,29 @@ static float *static_partials(hipStream_t stream, const char **why) {
 // ---- the same two passes over several gradient tensors at once ------------------------------------
 // A model whose gradients are separate allocations is scanned tensor by tensor otherwise: the 291 tensors of a
 // 6.74 B-parameter model cost 2.35 ms (flag) / 3.46 ms (flag and sum of squares, two launches each) against
-// 1.8 / 1.9 ms for one flat buffer, all of the difference launches; here 1.92 / 1.96 ms.  Up to kScanBatch tensors
+// 1.8 / 1.9 ms for one flat buffer, all of the difference launches; here 1.88 / 1.96 ms.  Up to kScanBatch tensors
 // travel in the kernel arguments; tiles are numbered through the tensors, a workgroup finds its tensor from the
 // table in the arguments, and the first tile of a tensor also takes that tensor's elements in front of and behind
 // its 16-byte vectors.  The partial sums are one per tile, as in the single-tensor kernel.
 constexpr int kScanBatch = 64;
 // Vectors per lane of the flag-only pass: the search in front makes a workgroup's start longer than the
-// single-tensor kernel's, and two vectors spread it (1 / 2 / 4 / 8 vectors: 65 / 87 / 81 / 86 % of the HBM
-// peak over the 291 gradient tensors of a 6.74 B-parameter model).
+// single-tensor kernel's, and two vectors spread it (1 / 2 / 3 vectors: 48 / 89.5 / 85.5 % of the HBM peak over
+// the 291 gradient tensors of a 6.74 B-parameter model).
 constexpr int kScanMultiUnroll = 2;
-// first_tile[k]: number of the first tile of tensor k; first_tile[count] = tiles of the launch; entries behind it
-// hold 0xFFFFFFFF.  Every tensor has at least one tile, so the used entries rise strictly.  every_4th[j] repeats
-// first_tile[4 j]: a workgroup finds its tensor with two rounds of scalar loads (16 entries, then the 4 between
-// two of them) instead of the six dependent ones of a bisection - the search runs in front of the workgroup's
-// only loads of data, so every round of it is time the memory pipeline of that workgroup's slot stands idle.
+// Tensors travel in sets of four: first[i] is the number of the first tile of the set's tensor i (0xFFFFFFFF
+// behind the last tensor of the launch; every tensor has at least one tile, so the used entries rise strictly),
+// and every_4th[j] repeats four[j].first[0].  A workgroup finds its tensor with two rounds of scalar loads - the
+// 16 entries of every_4th, then one set with its pointers and counts - instead of the six dependent loads of a
+// bisection and a seventh for pointer and count: the search runs in front of the workgroup's only loads of data,
+// so every round of it is time in which that workgroup's share of the memory pipeline stands idle.
+struct ScanFour {
+    uint32_t first[4];
+    const uint16_t *g[4];
+    int64_t n[4];
+};
 struct ScanBatch {
-    const uint16_t *g[kScanBatch];
-    int64_t n[kScanBatch];
-    uint32_t first_tile[kScanBatch + 4];
+    ScanFour four[kScanBatch / 4];
     uint32_t every_4th[kScanBatch / 4];
-    int32_t count;
 };
 
 template <typename T, bool STATS>
@@ -257,13 +260,14 @@ __global__ __launch_bounds__(kScanThreads) void scan_multi_kernel(ScanBatch batc
     int group = -1;                                    // every_4th[group] <= blockIdx.x < every_4th[group + 1]
 #pragma unroll
     for (int j = 0; j < kScanBatch / 4; j++) group += batch.every_4th[j] <= blockIdx.x ? 1 : 0;
-    const uint32_t *four = batch.first_tile + 4 * group;
-    const uint32_t f0 = four[0], f1 = four[1], f2 = four[2], f3 = four[3];
+    const ScanFour &set = batch.four[group];
+    const uint32_t f0 = set.first[0], f1 = set.first[1], f2 = set.first[2], f3 = set.first[3];
+    const uint16_t *g0 = set.g[0], *g1 = set.g[1], *g2 = set.g[2], *g3 = set.g[3];
+    const int64_t n0 = set.n[0], n1 = set.n[1], n2 = set.n[2], n3 = set.n[3];
     const int within = (f1 <= blockIdx.x ? 1 : 0) + (f2 <= blockIdx.x ? 1 : 0) + (f3 <= blockIdx.x ? 1 : 0);
-    const int lo = 4 * group + within;
     const uint32_t first = within == 0 ? f0 : within == 1 ? f1 : within == 2 ? f2 : f3;
-    const uint16_t *g = batch.g[lo];
-    const int64_t n = batch.n[lo];
+    const uint16_t *g = within == 0 ? g0 : within == 1 ? g1 : within == 2 ? g2 : g3;
+    const int64_t n = within == 0 ? n0 : within == 1 ? n1 : within == 2 ? n2 : n3;
     const uint32_t tile = blockIdx.x - first;
     int64_t head = (int64_t)(((16 - ((uintptr_t)g & 15u)) & 15u) / 2);
     if (head > n) head = n;
@@ -333,13 +337,17 @@ static int scan_multi(int32_t count, const bmt_scan_tensor *tensors, void *sumsq
         if (tensors[k].n / per_tile + 1 > 0x3FFFFFFF) return fail(-1, "grad_stats_multi_launcher: tensor too large for one launch");
     }
     ScanBatch batch;
-    batch.count = 0;
-    batch.first_tile[0] = 0;
+    int held = 0;                                      // tensors in the batch
+    uint32_t tiles_held = 0;                           // and their tiles
     auto flush = [&]() -> hipError_t {
-        if (batch.count == 0) return hipSuccess;
-        const uint32_t tiles = batch.first_tile[batch.count];
-        for (int k = batch.count + 1; k < kScanBatch + 4; k++) batch.first_tile[k] = 0xFFFFFFFFu;
-        for (int j = 0; j < kScanBatch / 4; j++) batch.every_4th[j] = batch.first_tile[4 * j];
+        if (held == 0) return hipSuccess;
+        for (int k = held; k < kScanBatch; k++) {      // behind the last tensor: never found, never dereferenced
+            batch.four[k / 4].first[k % 4] = 0xFFFFFFFFu;
+            batch.four[k / 4].g[k % 4] = nullptr;
+            batch.four[k / 4].n[k % 4] = 0;
+        }
+        for (int j = 0; j < kScanBatch / 4; j++) batch.every_4th[j] = batch.four[j].first[0];
+        const uint32_t tiles = tiles_held;
         if (sumsq) {
             hipLaunchKernelGGL((scan_multi_kernel<T, true>), dim3(tiles), dim3(kScanThreads), 0, (hipStream_t)stream, batch,
                                (uint8_t *)flag, (float *)workspace);
@@ -349,8 +357,8 @@ static int scan_multi(int32_t count, const bmt_scan_tensor *tensors, void *sumsq
             hipLaunchKernelGGL((scan_multi_kernel<T, false>), dim3(tiles), dim3(kScanThreads), 0, (hipStream_t)stream, batch,
                                (uint8_t *)flag, (float *)nullptr);
         }
-        batch.count = 0;
-        batch.first_tile[0] = 0;
+        held = 0;
+        tiles_held = 0;
         return hipGetLastError();
     };
     for (int32_t k = 0; k < count; k++) {
@@ -362,15 +370,15 @@ static int scan_multi(int32_t count, const bmt_scan_tensor *tensors, void *sumsq
         const int64_t nvec = (n - head) / 8;
         int64_t tiles = (nvec * 8 + per_tile - 1) / per_tile;
         if (tiles < 1) tiles = 1;
-        if (batch.count == kScanBatch || (int64_t)batch.first_tile[batch.count] + tiles > 0x7FFFFFFF) {
+        if (held == kScanBatch || (int64_t)tiles_held + tiles > 0x7FFFFFFF) {
             hipError_t e = flush();
             if (e != hipSuccess) return fail((int)e, who, e);
         }
-        const int c = batch.count;
-        batch.g[c] = (const uint16_t *)tensors[k].g_16;
-        batch.n[c] = n;
-        batch.first_tile[c + 1] = batch.first_tile[c] + (uint32_t)tiles;
-        batch.count = c + 1;
+        batch.four[held / 4].first[held % 4] = tiles_held;
+        batch.four[held / 4].g[held % 4] = (const uint16_t *)tensors[k].g_16;
+        batch.four[held / 4].n[held % 4] = n;
+        tiles_held += (uint32_t)tiles;
+        held++;
     }
     hipError_t e = flush();
     return e == hipSuccess ? 0 : fail((int)e, who, e);
