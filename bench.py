@@ -321,7 +321,7 @@ def other_workloads(torch, dev, LF, OF, iters=20):
         "ms": round(stats[0], 4), "ms_median": round(stats[1], 4), "ms_min": round(stats[2], 4),
         "rows_per_s": round(rows / (stats[0] * 1e-3), 1),
         "what": "FusedCrossEntropy(ignore_index=-100)(x, t).backward(): the two kernels plus allocation of the 1 GB softmax / "
-                "gradient tensor, the int32 cast of the targets, mask, mean and autograd"}
+                "gradient tensor, the int32 cast of the targets, the mean over the rows that are not ignored (one launch each way) and autograd"}
     x.grad = None
     del x, t64
     torch.cuda.empty_cache()
@@ -507,7 +507,7 @@ def full_model_side_measurements(torch, OF, p16, grad, p32, mom, var, iters=5):
     return out
 
 
-KERNEL_SOURCES = ("adam.hip", "cross_entropy.hip", "has_inf_nan.hip", "bmt_device.h", "bmt_host.h")
+KERNEL_SOURCES = ("adam.hip", "cross_entropy.hip", "has_inf_nan.hip", "loss_reduce.hip", "bmt_device.h", "bmt_host.h")
 
 
 def kernel_sources_digest():

@@ -46,6 +46,8 @@ _SIGNATURES = {
     "grad_stats_fp16_launcher": [_i64, _p, _p, _p, _p, _p],
     "grad_stats_bf16_launcher": [_i64, _p, _p, _p, _p, _p],
     "grad_stats_noalloc_launcher": [_i64, _p, _i32, _p, _p, _p],
+    "cross_entropy_reduce_forward_launcher": [_i64, _p, _p, _p, _i32, _i32, _i32, _p, _p, _p],
+    "cross_entropy_reduce_backward_launcher": [_i64, _p, _p, _i32, _i32, _i32, _p, _p, _p, _p],
 }
 
 _lib.bmt_hip_last_error.restype = ctypes.c_char_p

@@ -97,3 +97,38 @@ def fused_softmax_inplace(logits: torch.Tensor, max_logits: torch.Tensor, sum_ex
     launcher = _pick("fused_softmax_inplace", logits.dtype,
                      C.fused_softmax_inplace_fp16_launcher, C.fused_softmax_inplace_bf16_launcher)
     launcher(m, n, logits.data_ptr(), max_logits.data_ptr(), sum_exp_logits.data_ptr(), _current_stream())
+
+
+def loss_reduce_forward(losses: torch.Tensor, target: torch.Tensor, weight, n_classes: int, ignore_index: int,
+                        mean: bool, result: torch.Tensor, weight_sum: torch.Tensor) -> None:
+    """``result = sum_r w_r * losses[r]`` (divided by ``weight_sum = sum_r w_r`` when ``mean``) with
+    ``w_r = 0`` for ignored rows and otherwise ``weight[target[r]]`` (1 without ``weight``): the reduction that
+    bmtrain/loss/cross_entropy.py:243-260 writes in torch operations, in one launch."""
+    for name, t in (("losses", losses), ("target", target), ("result", result), ("weight_sum", weight_sum)):
+        assert _on_gpu(t), f"{name} must be contiguous and on cuda"
+    assert losses.dtype == torch.float32 and result.dtype == torch.float32 and weight_sum.dtype == torch.float32
+    assert target.dtype == torch.int32, "target must be an int tensor"
+    assert target.numel() == losses.numel(), "target and losses must have the same number of elements"
+    if weight is not None:
+        assert _on_gpu(weight) and weight.dtype == torch.float32 and weight.numel() == n_classes, \
+            "weight must be a contiguous float tensor of n_classes elements on cuda"
+    C.cross_entropy_reduce_forward_launcher(losses.numel(), losses.data_ptr(), target.data_ptr(),
+                                            weight.data_ptr() if weight is not None else 0, n_classes, ignore_index,
+                                            int(mean), result.data_ptr(), weight_sum.data_ptr(), _current_stream())
+
+
+def loss_reduce_backward(target: torch.Tensor, weight, n_classes: int, ignore_index: int, mean: bool,
+                         weight_sum: torch.Tensor, upstream: torch.Tensor, grad_rows: torch.Tensor) -> None:
+    """``grad_rows[r] = (upstream / weight_sum if mean else upstream) * w_r``: what autograd derives from the
+    torch operations of bmtrain/loss/cross_entropy.py:243-260, in one launch."""
+    for name, t in (("target", target), ("weight_sum", weight_sum), ("upstream", upstream), ("grad_rows", grad_rows)):
+        assert _on_gpu(t), f"{name} must be contiguous and on cuda"
+    assert upstream.dtype == torch.float32 and upstream.numel() == 1, "upstream must be one float"
+    assert weight_sum.dtype == torch.float32 and grad_rows.dtype == torch.float32
+    assert target.dtype == torch.int32 and target.numel() == grad_rows.numel()
+    if weight is not None:
+        assert _on_gpu(weight) and weight.dtype == torch.float32 and weight.numel() == n_classes
+    C.cross_entropy_reduce_backward_launcher(target.numel(), target.data_ptr(),
+                                             weight.data_ptr() if weight is not None else 0, n_classes, ignore_index,
+                                             int(mean), weight_sum.data_ptr(), upstream.data_ptr(), grad_rows.data_ptr(),
+                                             _current_stream())

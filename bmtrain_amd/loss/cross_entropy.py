@@ -37,6 +37,36 @@ class OpFusedCrossEntropy(torch.autograd.Function):
         return (softmax, None, None)
 
 
+class OpLossReduce(torch.autograd.Function):
+    """``sum`` / ``mean`` reduction of per-row losses with ignored rows and class weights — the torch expressions
+    of bmtrain/loss/cross_entropy.py:243-260 (mask or gathered weights, product, two sums, quotient; about ten
+    launches forward and six backward for [N]-sized tensors) as one launch each way.  The gradient per row is the
+    same two fp32 operations autograd performs; the loss differs from the torch expression only by the order in
+    which the rows are added (here: in double, then rounded once)."""
+
+    MAX_ROWS = 1 << 20      # the forward launch is one workgroup
+
+    @staticmethod
+    def forward(ctx, losses: torch.Tensor, target: torch.Tensor, weight, n_classes: int, ignore_index: int, mean: bool):
+        losses = losses.contiguous()
+        result = torch.empty((), device=losses.device, dtype=torch.float)
+        weight_sum = torch.empty((), device=losses.device, dtype=torch.float)
+        F.loss_reduce_forward(losses, target, weight, n_classes, ignore_index, mean, result, weight_sum)
+        ctx.args = (n_classes, ignore_index, mean)
+        ctx.weight = weight
+        ctx.save_for_backward(target, weight_sum)
+        return result
+
+    @staticmethod
+    def backward(ctx, upstream: torch.Tensor):
+        target, weight_sum = ctx.saved_tensors
+        n_classes, ignore_index, mean = ctx.args
+        upstream = upstream.float().contiguous()
+        grad_rows = torch.empty(target.numel(), device=target.device, dtype=torch.float)
+        F.loss_reduce_backward(target, ctx.weight, n_classes, ignore_index, mean, weight_sum, upstream, grad_rows)
+        return (grad_rows, None, None, None, None, None)
+
+
 def _tp_all_reduce(t: torch.Tensor, op: str) -> torch.Tensor:
     """All-reduce over the tensor-parallel group.  With a group of one (the only case this
     single-GPU package runs) the reduction is the identity; a larger group needs the
@@ -126,8 +156,21 @@ class FusedCrossEntropy(torch.nn.Module):
         self.reduction = reduction
         self.label_smoothing = label_smoothing
         self.parallel = parallel
+        # sum / mean of the per-row losses in one launch each way (OpLossReduce); False: the reference's torch operations
+        self.fused_reduction = True
+
+    def _can_fuse(self, losses: torch.Tensor, target: torch.Tensor) -> bool:
+        if not losses.is_cuda or losses.dtype != torch.float32 or losses.numel() > OpLossReduce.MAX_ROWS:
+            return False
+        if target.dim() != 1 or target.numel() != losses.numel():
+            return False
+        w = self.weight
+        if w is not None and self.parallel:     # class weights are indexed by the global class, not by this rank's slice
+            return False
+        return w is None or (w.is_cuda and w.device == losses.device and not w.requires_grad and w.is_floating_point())
 
     def forward(self, input: torch.Tensor, target: torch.Tensor) -> torch.Tensor:
+        target32 = None
         if self.parallel:
             ret = VPFusedCrossEntropy.apply(input, target.long())
         elif input.dtype == torch.float32:
@@ -135,12 +178,19 @@ class FusedCrossEntropy(torch.nn.Module):
                 input, target.long(), weight=self.weight, ignore_index=self.ignore_index,
                 reduction=self.reduction, label_smoothing=self.label_smoothing)
         else:
-            ret = OpFusedCrossEntropy.apply(input, target.int(), self.ignore_index)
+            target32 = target.int().contiguous()
+            ret = OpFusedCrossEntropy.apply(input, target32, self.ignore_index)
+
+        if self.weight is not None and (self.weight.dim() != 1 or self.weight.size(0) != input.size(1)):
+            raise ValueError("weight should be a 1D tensor of size C")
+        if self.fused_reduction and self.reduction in ("sum", "mean") and self._can_fuse(ret, target):
+            weight = None if self.weight is None else self.weight.detach().float().contiguous()
+            if target32 is None:
+                target32 = target.int().contiguous()
+            return OpLossReduce.apply(ret, target32, weight, input.size(1), self.ignore_index, self.reduction == "mean")
 
         ignored = target == self.ignore_index
         if self.weight is not None:
-            if self.weight.dim() != 1 or self.weight.size(0) != input.size(1):
-                raise ValueError("weight should be a 1D tensor of size C")
             w = self.weight[torch.where(ignored, 0, target)].float()
             w[ignored] = 0
         else:

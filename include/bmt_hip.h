@@ -170,6 +170,25 @@ BMT_API int fused_softmax_inplace_bf16_launcher(int32_t m, int32_t n, void *logi
                                         const void *sum_exp_logits, void *stream);
 
 /*
+ * cross_entropy_reduce_{forward,backward}_launcher — no counterpart in the reference's extension: the
+ * reduction of the per-row losses that FusedCrossEntropy.forward spells out in torch operations
+ * (bmtrain/loss/cross_entropy.py:243-260) and its autograd backward, one launch each.
+ *   w_r = target[r] == ignore_index ? 0 : (weight ? weight[target[r]] : 1)       (weight: float[n_classes] or NULL;
+ *                                                                                 a class outside the table weighs 0)
+ *   forward:  weight_sum[0] = sum_r w_r;  result[0] = sum_r w_r * losses[r], divided by weight_sum[0] when `mean`
+ *   backward: grad_rows[r] = (mean ? upstream[0] / weight_sum[0] : upstream[0]) * w_r
+ * losses, grad_rows: float[m]; target: int32[m]; result, weight_sum, upstream: one float each, all on the device.
+ * The sums are taken in double in a fixed order and rounded to float once; the forward launch is one workgroup
+ * (meant for row counts up to about a million).
+ */
+BMT_API int cross_entropy_reduce_forward_launcher(int64_t m, const void *losses, const void *target, const void *weight,
+                                                  int32_t n_classes, int32_t ignore_index, int32_t mean, void *result,
+                                                  void *weight_sum, void *stream);
+BMT_API int cross_entropy_reduce_backward_launcher(int64_t m, const void *target, const void *weight, int32_t n_classes,
+                                                   int32_t ignore_index, int32_t mean, const void *weight_sum,
+                                                   const void *upstream, void *grad_rows, void *stream);
+
+/*
  * adam_{fp16,bf16}_multi_launcher — no counterpart in the reference's extension, which is called once
  * per parameter tensor from the Python loop of AdamOptimizer.step (bmtrain/optim/adam.py:72-159).  Steps
  * `count` tensors that share their hyper-parameters (same group, same step count) in as few launches as

@@ -355,6 +355,81 @@ def test_module_with_class_weights_and_ignored_targets(dtype):
             torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-4 if reduction == "none" else 1.0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_reduction_against_the_torch_expressions(dtype):
+    """FusedCrossEntropy reduces the per-row losses with one launch each way (OpLossReduce) where
+    bmtrain/loss/cross_entropy.py:243-260 uses torch operations; with `fused_reduction = False` the module runs those
+    operations.  Same rows, same targets: the loss agrees to 1e-6 relative (only the order of the additions differs, torch adds in fp32;
+    the fused sums are checked against float64 arithmetic below), the logits' gradient is bit-identical - except under
+    `mean` with class weights, where the divisor is a rounded sum of weights that may differ in its last bit and the
+    gradient then differs by one step of the 16-bit type on a few elements - for sum and mean, with and without class
+    weights (fp32 and 16-bit), with no, some and all rows ignored, for row counts around the kernel's strides, and with
+    an upstream factor as a loss scale gives."""
+    torch.manual_seed(11)
+    for m, C in ((1, 17), (7, 100), (1000, 257), (1023, 64), (1025, 64), (4097, 1000), (16384, 512)):
+        x = (torch.randn(m, C, device="cuda") * 2).to(dtype)
+        for ignored in ("none", "some", "all"):
+            tgt = torch.randint(0, C, (m,), device="cuda")
+            if ignored == "some":
+                tgt[torch.rand(m, device="cuda") < 0.3] = -100
+            elif ignored == "all":
+                tgt[:] = -100
+            for weight in (None, torch.rand(C, device="cuda") + 0.5, (torch.rand(C, device="cuda") + 0.5).to(dtype)):
+                for reduction in ("mean", "sum"):
+                    for scale in (1.0, 32768.0):
+                        results = []
+                        for fused in (True, False):
+                            module = FusedCrossEntropy(weight=weight, reduction=reduction)
+                            module.fused_reduction = fused
+                            xi = x.clone().requires_grad_()
+                            loss = module(xi, tgt)
+                            (loss * scale).backward()
+                            results.append((loss.detach(), xi.grad))
+                        (la, ga), (lb, gb) = results
+                        assert la.dtype == lb.dtype == torch.float32 and la.shape == lb.shape == ()
+                        case = (m, C, ignored, None if weight is None else weight.dtype, reduction, scale)
+                        if ignored == "all" and reduction == "mean":
+                            assert torch.isnan(la) and torch.isnan(lb), case          # 0 / 0, as in the reference
+                            assert torch.isnan(ga).all() and torch.isnan(gb).all(), case
+                            continue
+                        assert abs(la.item() - lb.item()) <= 1e-6 * abs(lb.item()) + 1e-30, case
+                        if weight is not None and reduction == "mean":
+                            # the divisor is itself a rounded sum of weights here: it may differ in its last bit
+                            steps = (ga.view(torch.int16).int() - gb.view(torch.int16).int()).abs()
+                            assert steps.max().item() <= 1 and (steps > 0).float().mean().item() < 0.02, case
+                        else:
+                            assert torch.equal(ga.view(torch.int16), gb.view(torch.int16)), case
+    # the launchers by themselves against float64 arithmetic, also beyond the 4 x 1024 rows of one pass of the loop
+    from bmtrain_amd.loss import _function as LF
+    for m in (0, 1, 4095, 4096, 4097, 100_000):
+        losses = torch.rand(m, device="cuda") * 12
+        tgt = torch.randint(0, 50, (m,), device="cuda", dtype=torch.int32)
+        tgt[::7] = -1
+        weight = torch.rand(50, device="cuda") + 0.1
+        for w in (None, weight):
+            for mean in (False, True):
+                result, wsum = torch.empty((), device="cuda"), torch.empty((), device="cuda")
+                LF.loss_reduce_forward(losses, tgt, w, 50, -1, mean, result, wsum)
+                wr = ((tgt != -1).float() if w is None else torch.where(tgt != -1, weight[tgt.clamp(min=0).long()], 0.0))
+                exact_s = (wr * losses).double().sum().item()
+                exact_w = wr.double().sum().item()
+                assert abs(wsum.item() - exact_w) <= 6e-8 * exact_w
+                if exact_w == 0 and mean:            # no row counts: 0 / 0, as in the reference
+                    assert torch.isnan(result)
+                    continue
+                want = exact_s / exact_w if mean else exact_s
+                assert abs(result.item() - want) <= 2e-7 * abs(want), (m, mean)
+                up = torch.full((), 3.0, device="cuda")
+                rows = torch.empty(m, device="cuda")
+                LF.loss_reduce_backward(tgt, w, 50, -1, mean, wsum, up, rows)
+                assert torch.equal(rows, (up / wsum if mean else up) * wr)
+    # a class outside the weight table weighs nothing instead of being read
+    tgt = torch.tensor([3, 50, -7, 2], device="cuda", dtype=torch.int32)
+    result, wsum = torch.empty((), device="cuda"), torch.empty((), device="cuda")
+    LF.loss_reduce_forward(torch.ones(4, device="cuda"), tgt, weight, 50, -100, False, result, wsum)
+    assert wsum.item() == (weight[3] + weight[2]).item()
+
+
 def test_module_contract():
     x = torch.randn(8, 16, device="cuda")
     tgt = torch.randint(0, 16, (8,), device="cuda")
