@@ -53,17 +53,16 @@ class OpLossReduce(torch.autograd.Function):
         weight_sum = torch.empty((), device=losses.device, dtype=torch.float)
         F.loss_reduce_forward(losses, target, weight, n_classes, ignore_index, mean, result, weight_sum)
         ctx.args = (n_classes, ignore_index, mean)
-        ctx.weight = weight
-        ctx.save_for_backward(target, weight_sum)
+        ctx.save_for_backward(target, weight_sum, weight)
         return result
 
     @staticmethod
     def backward(ctx, upstream: torch.Tensor):
-        target, weight_sum = ctx.saved_tensors
+        target, weight_sum, weight = ctx.saved_tensors
         n_classes, ignore_index, mean = ctx.args
         upstream = upstream.float().contiguous()
         grad_rows = torch.empty(target.numel(), device=target.device, dtype=torch.float)
-        F.loss_reduce_backward(target, ctx.weight, n_classes, ignore_index, mean, weight_sum, upstream, grad_rows)
+        F.loss_reduce_backward(target, weight, n_classes, ignore_index, mean, weight_sum, upstream, grad_rows)
         return (grad_rows, None, None, None, None, None)
 
 
