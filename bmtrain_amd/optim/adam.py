@@ -97,41 +97,58 @@ class AdamOptimizer(torch.optim.Optimizer):
     supports_grad_coef = True
 
     @torch.no_grad()
-    def step(self, closure=None, scale=1, grad_coef=None):
+    def step(self, closure=None, scale=1, grad_coef=None, _plan=None):
         """One optimisation step; ``scale`` is the loss scale the gradients carry.  ``grad_coef`` (a 0-dim
         tensor or float below one) clips on the fly: each gradient enters as if it had been multiplied in
         place by it — for 16-bit gradients with the factor rounded to their dtype and the product rounded
-        back, as the in-place multiplication does on the GPU — but the gradient tensors are left alone."""
+        back, as the in-place multiplication does on the GPU — but the gradient tensors are left alone.
+        ``_plan``: what ``plan_step`` returned for the same arguments a moment ago (OptimManager prepares the
+        step while the overflow scan is still running on the GPU)."""
         loss = None
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
+        for action in (self.plan_step(scale, grad_coef) if _plan is None else _plan):
+            action()
+        return loss
 
+    @torch.no_grad()
+    def plan_step(self, scale=1, grad_coef=None, create_state=True):
+        """The host side of a step — which tensors go into which launch, with which step count and learning
+        rate — as a list of calls that ``step`` then only has to make.  Nothing of the optimizer's state changes
+        here except that parameters seen for the first time get their state; with ``create_state=False`` not
+        even that: None is returned instead of a plan when a parameter has no state yet (a step that may still be
+        called off must not copy parameters into master weights).  A plan is only good for a step taken right
+        away, before anybody touches parameters, gradients or state."""
+        actions = []
         for group in self.param_groups:
             beta1, beta2 = group["betas"][0], group["betas"][1]
+            eps, weight_decay = group["eps"], group["weight_decay"]
             active = [p for p in group["params"] if p.grad is not None and p.requires_grad]
             for p in active:
                 check_grad(p)
-            self._init_states([p for p in active if len(self.state[p]) == 0])
+            fresh = [p for p in active if len(self.state[p]) == 0]
+            if fresh and not create_state:
+                return None
+            self._init_states(fresh)
 
             half = []     # 16-bit work: (param_fp32, param, grad, exp_avg, exp_avg_sq, step, lr)
+            counted = []  # their states: the step count goes up when the step is taken
             for p in active:
                 state = self.state[p]
                 grad = -p.grad if wants_maximize(group) else p.grad
                 if p.dtype == torch.float32:
                     # hold_steps is tested before the increment on this path (adam.py:137).
                     lr = 0.0 if state["step"] < self._hold_steps else group["lr"]
-                    if grad_coef is not None:
-                        grad = grad * grad_coef
-                    torch_adam_fp32(p, grad / scale, state["exp_avg"], state["exp_avg_sq"], state["step"],
-                                    beta1=beta1, beta2=beta2, lr=lr, weight_decay=group["weight_decay"],
-                                    eps=group["eps"])
-                    state["step"] += 1
+                    actions.append(self._fp32_action(p, grad, state, lr, scale, grad_coef, beta1, beta2, eps, weight_decay))
                 else:
                     # ... and after the increment on the fused path (adam.py:145,155).
-                    state["step"] += 1
-                    lr = 0.0 if state["step"] < self._hold_steps else group["lr"]
-                    half.append((state["_param_fp32"], p, grad, state["exp_avg"], state["exp_avg_sq"], state["step"], lr))
+                    step = state["step"] + 1
+                    lr = 0.0 if step < self._hold_steps else group["lr"]
+                    half.append((state["_param_fp32"], p, grad, state["exp_avg"], state["exp_avg_sq"], step, lr))
+                    counted.append(state)
+            if counted:
+                actions.append(self._count_action(counted))
 
             # 16-bit parameters that can share launches: (dtype, step, lr) -> tensors.
             batches, singles = {}, []
@@ -153,15 +170,45 @@ class AdamOptimizer(torch.optim.Optimizer):
                 singles.extend(w for w in batches[key] if w[1].numel() >= self.alone_from)
                 batches[key] = [w for w in batches[key] if w[1].numel() < self.alone_from]
             for p32, p, grad, m, v, step, lr in singles:
-                if coef16:                 # not contiguous: clip a copy of the gradient eagerly
-                    grad = grad * torch.as_tensor(grad_coef, dtype=torch.float32, device=grad.device)
-                fused = F.adam_fp16 if p.dtype == torch.float16 else F.adam_bf16
-                fused(p32, p, grad, m, v, beta1, beta2, group["eps"], lr, scale, group["weight_decay"], step)
-            batches = {key: [w[:5] for w in items] for key, items in batches.items() if items}
-            for (dtype, step, lr), tensors in batches.items():
-                F.adam_multi(tensors, beta1, beta2, group["eps"], lr, scale, group["weight_decay"], step,
-                             grad_coef=coef16.get(dtype, 1.0))
-        return loss
+                actions.append(self._single_action(p32, p, grad, m, v, step, lr, scale, grad_coef if coef16 else None,
+                                                   beta1, beta2, eps, weight_decay))
+            for (dtype, step, lr), items in batches.items():
+                if items:
+                    actions.append(self._multi_action([w[:5] for w in items], step, lr, scale, coef16.get(dtype, 1.0),
+                                                      beta1, beta2, eps, weight_decay))
+        return actions
+
+    @staticmethod
+    def _count_action(states):
+        def run():
+            for state in states:
+                state["step"] += 1
+        return run
+
+    @staticmethod
+    def _multi_action(tensors, step, lr, scale, coef, beta1, beta2, eps, weight_decay):
+        def run():
+            F.adam_multi(tensors, beta1, beta2, eps, lr, scale, weight_decay, step, grad_coef=coef)
+        return run
+
+    @staticmethod
+    def _fp32_action(p, grad, state, lr, scale, grad_coef, beta1, beta2, eps, weight_decay):
+        def run():
+            g = grad if grad_coef is None else grad * grad_coef
+            torch_adam_fp32(p, g / scale, state["exp_avg"], state["exp_avg_sq"], state["step"],
+                            beta1=beta1, beta2=beta2, lr=lr, weight_decay=weight_decay, eps=eps)
+            state["step"] += 1
+        return run
+
+    @staticmethod
+    def _single_action(p32, p, grad, m, v, step, lr, scale, grad_coef, beta1, beta2, eps, weight_decay):
+        def run():
+            g = grad
+            if grad_coef is not None:      # not contiguous: clip a copy of the gradient eagerly
+                g = grad * torch.as_tensor(grad_coef, dtype=torch.float32, device=grad.device)
+            fused = F.adam_fp16 if p.dtype == torch.float16 else F.adam_bf16
+            fused(p32, p, g, m, v, beta1, beta2, eps, lr, scale, weight_decay, step)
+        return run
 
     def get_avg_delta():
         raise NotImplementedError(

@@ -42,17 +42,26 @@ def _fingerprint(g):
     return (g.data_ptr(), g.numel(), g.dtype, g._version)
 
 
+def launch_overflow_scan(param_groups, known=None, flag=None):
+    """Starts the scan of check_overflow and returns the flag it writes (None when there is nothing to scan), without
+    waiting for it.  `known` may carry the verdict of an earlier pass over gradients: a pair (flag tensor,
+    {fingerprint}); gradients found in it unchanged are not read again.  `flag`: a flag to go on with (it is sticky)."""
+    grads = _scanned_grads(param_groups)
+    if not grads:
+        return flag
+    if known is not None and all(_fingerprint(g) in known[1] for g in grads):
+        return known[0] if flag is None else torch.maximum(flag, known[0])
+    if flag is None:
+        flag = torch.zeros(1, dtype=torch.uint8, device="cuda")[0]
+    _scan(grads, None, flag)
+    return flag
+
+
 def check_overflow(param_groups, known=None):
     """Raises OverflowError when any non-fp32 gradient holds an inf or NaN
-    (optim_manager.py:9-21).  `known` may carry the verdict of an earlier pass over gradients:
-    a pair (flag tensor, {fingerprint}); gradients found in it unchanged are not read again."""
-    grads = _scanned_grads(param_groups)
-    if known is not None and all(_fingerprint(g) in known[1] for g in grads):
-        flag = known[0]
-    else:
-        flag = torch.zeros(1, dtype=torch.uint8, device="cuda")[0]
-        _scan(grads, None, flag)
-    if flag > 0:
+    (optim_manager.py:9-21)."""
+    flag = launch_overflow_scan(param_groups, known)
+    if flag is not None and flag > 0:
         raise OverflowError("Gradient overflow")
 
 
@@ -142,21 +151,32 @@ class OptimManager:
             return None
         return self._known_overflow
 
-    def _overflowed(self) -> bool:
+    def _overflowed(self, meanwhile=None) -> bool:
+        """One sticky flag over the gradients of all optimizers, read once.  `meanwhile` is called between the
+        launches and the read: host work done there runs while the GPU scans."""
         known = self._verdict_usable()
+        flag = None
         for optimizer in self.optimizers:
-            try:
-                check_overflow(optimizer.param_groups, known)
-            except OverflowError:
-                self._known_overflow = None
-                return True
+            flag = launch_overflow_scan(optimizer.param_groups, known, flag)
         self._known_overflow = None
-        return False
+        if meanwhile is not None:
+            meanwhile()
+        return flag is not None and bool(flag > 0)
 
     def step(self):
         """Skips the step and lowers the scale on overflow; otherwise steps every optimizer
         and scheduler and raises the scale after ``loss_scale_steps`` clean steps."""
-        if self.loss_scale_enabled and self._overflowed():
+        pending = None if self._pending_clip is None else self._pending_clip[0]
+        plans = {}
+
+        def plan_steps():       # the optimizers' host-side preparation; under loss scaling it overlaps the overflow scan
+            for optimizer in self.optimizers:
+                if getattr(optimizer, "_bmtrain_optimizer", False) and hasattr(optimizer, "plan_step"):
+                    plan = optimizer.plan_step(scale=self.loss_scale, grad_coef=pending, create_state=False)
+                    if plan is not None:
+                        plans[id(optimizer)] = plan
+
+        if self.loss_scale_enabled and self._overflowed(meanwhile=plan_steps):
             lowered = self.loss_scale / self.loss_scale_factor
             print("Gradient overflow, change scale from %lf to %lf" % (self.loss_scale, lowered))
             with torch.no_grad():
@@ -164,11 +184,12 @@ class OptimManager:
                     self._justify_scale(lowered)
                 self.zero_grad()
             return
-        pending = None if self._pending_clip is None else self._pending_clip[0]
         self._pending_clip = None
         self._clip_calls = 0
         for optimizer, lr_scheduler in zip(self.optimizers, self.lr_schedulers):
-            if pending is not None:
+            if id(optimizer) in plans:
+                optimizer.step(scale=self.loss_scale, grad_coef=pending, _plan=plans[id(optimizer)])
+            elif pending is not None:
                 optimizer.step(scale=self.loss_scale, grad_coef=pending)
             elif getattr(optimizer, "_bmtrain_optimizer", False):
                 optimizer.step(scale=self.loss_scale)

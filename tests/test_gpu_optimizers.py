@@ -526,6 +526,54 @@ def test_overflow_skips_the_step_and_halves_the_scale():
         bmt.optim.optim_manager.check_overflow([{"params": [p]}])
 
 
+def test_step_prepared_during_the_overflow_scan_is_the_step():
+    """OptimManager.step() lets the optimizers lay out their launches (plan_step) while the overflow scan runs and only
+    makes the calls once the flag has been read.  Through the manager and through optimizer.step() alone: the same
+    bits in parameters and state over several steps, for two parameter groups with their own hyper-parameters,
+    mixed fp32 / fp16 / bf16 parameters, hold_steps and maximize.  An overflow on the very first step leaves the
+    optimizer without state (no master copy of parameters that a caller may still load), and an overflow later
+    changes nothing but the moments' scale."""
+    def build():
+        torch.manual_seed(21)
+        ps = [torch.nn.Parameter(torch.randn(n, device="cuda").to(dt)) for n, dt in
+              ((5000, torch.bfloat16), (77, torch.float16), (4096, torch.bfloat16), (300, torch.float32), (1 << 16, torch.float16))]
+        opt = bmt.optim.AdamOptimizer([{"params": ps[:2], "lr": 1e-2, "weight_decay": 0.1, "betas": (0.8, 0.9)},
+                                       {"params": ps[2:], "lr": 3e-3, "eps": 1e-6, "maximize": True}], hold_steps=2)
+        return ps, opt
+    pa, oa = build()
+    pb, ob = build()
+    manager = bmt.optim.OptimManager(loss_scale=64.0, loss_scale_steps=10 ** 9)
+    manager.add_optimizer(oa)
+    # first step overflows: nothing is created
+    for p in pa:
+        p.grad = torch.full_like(p, float("inf") if p.dtype != torch.float32 else 0.0)
+    manager.step()
+    assert manager.loss_scale == 32.0 and all(len(oa.state[p]) == 0 for p in pa)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    for k in range(5):
+        grads = [(torch.randn(p.shape, device="cuda", generator=gen) * 32.0 * 1e-2).to(p.dtype) for p in pa]
+        for p, q, g in zip(pa, pb, grads):
+            p.grad, q.grad = g.clone(), g.clone()
+        if k == 3:          # an overflow in between: neither side steps; the moments kept in fp16 follow the new scale
+            pa[1].grad[5] = float("nan")
+            manager.step()
+            assert manager.loss_scale == 16.0
+            ob._on_justify_scale(32.0, 16.0)
+            continue
+        manager.step()
+        ob.step(scale=manager.loss_scale)
+    for p, q in zip(pa, pb):
+        assert torch.equal(p.detach().view(torch.uint8), q.detach().view(torch.uint8))
+        assert oa.state[p]["step"] == ob.state[q]["step"] == 4
+        for key in ("exp_avg", "exp_avg_sq"):
+            assert torch.equal(oa.state[p][key].view(torch.uint8), ob.state[q][key].view(torch.uint8)), key
+    # a plan is refused, not improvised, while a parameter has no state yet
+    pc, oc = build()
+    for p in pc:
+        p.grad = torch.zeros_like(p)
+    assert oc.plan_step(scale=1.0, create_state=False) is None and all(len(oc.state[p]) == 0 for p in pc)
+
+
 def test_hold_steps_and_maximize():
     p = torch.nn.Parameter(torch.ones(64, device="cuda").bfloat16())
     opt = bmt.optim.AdamOptimizer([p], lr=0.1, hold_steps=3)
