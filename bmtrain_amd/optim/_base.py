@@ -10,11 +10,22 @@ import torch.optim._functional as _torch_functional
 SUPPORTED_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
 
 
+def span(t):
+    """(storage address, first byte, byte behind the last, dtype) of a contiguous tensor; None otherwise."""
+    if not t.is_contiguous():
+        return None
+    begin = t.data_ptr()
+    return (t.untyped_storage().data_ptr(), begin, begin + t.numel() * t.element_size(), t.dtype)
+
+
+def span_follows(s, prev):
+    """True if the tensor of span `s` starts where the one of span `prev` ends, inside the same storage."""
+    return s is not None and prev is not None and s[1] == prev[2] and s[0] == prev[0] and s[3] == prev[3]
+
+
 def follows(t, prev):
     """True if contiguous tensor `t` starts where contiguous `prev` ends, inside the same storage."""
-    return (t.is_contiguous() and prev.is_contiguous() and t.dtype == prev.dtype
-            and t.data_ptr() == prev.data_ptr() + prev.numel() * prev.element_size()
-            and t.untyped_storage().data_ptr() == prev.untyped_storage().data_ptr())
+    return span_follows(span(t), span(prev))
 
 
 def flat_runs(tensors):
@@ -29,10 +40,13 @@ def flat_runs(tensors):
             out.append(run[0].as_strided((sum(t.numel() for t in run),), (1,)))
         run.clear()
 
+    last = None
     for t in tensors:
-        if run and not follows(t, run[-1]):
+        here = span(t)                     # every tensor is looked at once, not once from either side
+        if run and not span_follows(here, last):
             close()
         run.append(t)
+        last = here
     close()
     return out
 

@@ -14,20 +14,22 @@ the two moments are stored multiplied by the loss scale, which is why
 import torch
 
 from . import _function as F
-from ._base import check_grad, follows, remap_loaded_state, torch_adam_fp32, validate_hyper, wants_maximize
+from ._base import check_grad, follows, remap_loaded_state, span, span_follows, torch_adam_fp32, validate_hyper, wants_maximize
 
 
 def _adjacent_runs(work):
     """Splits 16-bit work items into maximal runs in which all five arrays of an item follow those of the
     item before and step count and learning rate agree."""
-    runs = []
+    runs, last = [], None
     for item in work:
+        here = [span(t) for t in item[:5]]
         prev = runs[-1][-1] if runs else None
         if (prev is not None and item[5] == prev[5] and item[6] == prev[6]
-                and all(follows(a, b) for a, b in zip(item[:5], prev[:5]))):
+                and all(span_follows(a, b) for a, b in zip(here, last))):
             runs[-1].append(item)
         else:
             runs.append([item])
+        last = here
     return runs
 
 
