@@ -275,7 +275,7 @@ class OptimManager:
         # verdict (it multiplies by a finite factor below one, or by zero when the norm itself is infinite);
         # step() reuses it for gradients that nobody has written to since.
         self._known_overflow = None
-        if scanned is not None:
+        if scanned is not None and self.reuse_overflow_verdict:
             self._known_overflow = (scanned[0][0], {_fingerprint(g) for g in scanned[1]})
         return total_norm / scale
 

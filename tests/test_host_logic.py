@@ -129,6 +129,36 @@ def test_runs_of_adjacent_tensors():
     assert _adjacent_runs([]) == []
 
 
+def test_a_planned_step_changes_nothing_until_it_is_taken():
+    """AdamOptimizer.plan_step on fp32 parameters (the path that runs without a GPU): planning touches neither
+    parameters nor state nor step counts, no plan is made for a parameter without state when told not to create it,
+    and taking the plan equals step()."""
+    import bmtrain_amd as bmt
+    torch.manual_seed(3)
+
+    def build():
+        torch.manual_seed(3)
+        ps = [torch.nn.Parameter(torch.randn(7)), torch.nn.Parameter(torch.randn(3, 4))]
+        for q in ps:
+            q.grad = torch.randn_like(q)
+        return ps, bmt.optim.AdamOptimizer([{"params": ps[:1], "lr": 1e-2}, {"params": ps[1:], "lr": 1e-3, "weight_decay": 0.1}])
+    pa, oa = build()
+    pb, ob = build()
+    assert oa.plan_step(scale=2.0, create_state=False) is None and all(len(oa.state[q]) == 0 for q in pa)
+    oa.step(scale=2.0)
+    ob.step(scale=2.0)
+    before = [q.detach().clone() for q in pa]
+    plan = oa.plan_step(scale=2.0, create_state=False)
+    assert plan is not None
+    assert all(torch.equal(q.detach(), b) for q, b in zip(pa, before)) and all(oa.state[q]["step"] == 1 for q in pa)
+    oa.step(scale=2.0, _plan=plan)
+    ob.step(scale=2.0)
+    for q, r in zip(pa, pb):
+        assert torch.equal(q.detach(), r.detach()) and oa.state[q]["step"] == ob.state[r]["step"] == 2
+        assert torch.equal(oa.state[q]["exp_avg"], ob.state[r]["exp_avg"])
+        assert torch.equal(oa.state[q]["exp_avg_sq"], ob.state[r]["exp_avg_sq"])
+
+
 def test_state_of_adjacent_parameters_is_allocated_back_to_back():
     flat = torch.zeros(64, dtype=torch.bfloat16)
     params = [torch.nn.Parameter(flat[0:16].view(4, 4)), torch.nn.Parameter(flat[16:24]), torch.nn.Parameter(flat[30:40]),
