@@ -66,10 +66,11 @@ def check_overflow(param_groups, known=None):
 
 
 def grad_rescale(param_groups, scale):
-    for group in param_groups:
-        for p in group["params"]:
-            if p.grad is not None and p.requires_grad:
-                p.grad /= scale
+    """`p.grad /= scale` for every parameter with a gradient (optim_manager.py:23-27), one launch per run of gradients
+    that lie back to back instead of one per parameter."""
+    grads = [p.grad for group in param_groups for p in group["params"] if p.grad is not None and p.requires_grad]
+    for g in flat_runs(grads):
+        g /= scale
 
 
 class OptimManager:

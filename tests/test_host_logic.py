@@ -159,6 +159,30 @@ def test_a_planned_step_changes_nothing_until_it_is_taken():
         assert torch.equal(oa.state[q]["exp_avg_sq"], ob.state[r]["exp_avg_sq"])
 
 
+def test_manager_unscales_the_gradients_of_a_foreign_optimizer():
+    """An optimizer that is not one of this package's gets its gradients divided by the loss scale before its own step
+    (optim_manager.py:23-27, :141-143): gradients that are views into one buffer are divided by one launch, with the
+    values of the per-parameter division; parameters that need no gradient are left alone."""
+    import bmtrain_amd as bmt
+    from bmtrain_amd.optim.optim_manager import grad_rescale
+    flat_p, flat_g = torch.randn(30), torch.randn(30) * 64
+    ps = [torch.nn.Parameter(flat_p[0:10]), torch.nn.Parameter(flat_p[10:24].view(2, 7)), torch.nn.Parameter(torch.randn(5)),
+          torch.nn.Parameter(torch.randn(4), requires_grad=False)]
+    ps[0].grad, ps[1].grad, ps[2].grad = flat_g[0:10], flat_g[10:24].view(2, 7), torch.randn(5) * 64
+    ps[3].grad = torch.ones(4)
+    want = [p.grad.clone() / 64 for p in ps[:3]]
+    untouched = flat_g[24:].clone()
+    grad_rescale([{"params": ps}], 64)
+    assert all(torch.equal(p.grad, w) for p, w in zip(ps, want)) and torch.equal(ps[3].grad, torch.ones(4))
+    assert torch.equal(flat_g[24:], untouched)
+    opt = torch.optim.SGD([p for p in ps if p.requires_grad], lr=0.5)
+    manager = bmt.optim.OptimManager(loss_scale=None)
+    manager.add_optimizer(opt)
+    before = [p.detach().clone() for p in ps[:3]]
+    manager.step()                                # no loss scaling: the foreign optimizer simply steps
+    assert all(torch.equal(p.detach(), b - 0.5 * w) for p, b, w in zip(ps, before, want))
+
+
 def test_state_of_adjacent_parameters_is_allocated_back_to_back():
     flat = torch.zeros(64, dtype=torch.bfloat16)
     params = [torch.nn.Parameter(flat[0:16].view(4, 4)), torch.nn.Parameter(flat[16:24]), torch.nn.Parameter(flat[30:40]),
