@@ -639,7 +639,7 @@ __global__ __launch_bounds__(kFlatThreads) void ce_flat_vec_kernel(
 }
 
 // ---- the element-wise kernels as a resident grid --------------------------------------------
-// Large arrays with rows of at least 8,192 elements (a multiple of 8, base 16-byte aligned) run the way the
+// Large arrays with rows of at least 8,192 elements run the way the
 // long Adam launches do (see adam.hip): one workgroup of 256 lanes per compute unit stays resident and works
 // through tiles of 1,024 vectors (16 KiB = four 4 KiB blocks, one load per lane and block) handed out by atomic
 // tickets, with the loads of the next tile in flight while the current one is computed and stored; the vector
@@ -666,11 +666,16 @@ constexpr int32_t kFlatStreamMinRow = kFlatStreamThreads * kFlatStreamVecs * 8;
 // workgroups of the running launch that have left
 static __device__ __align__(256) uint32_t flat_tickets[kFlatCounters * 1024];
 
-template <typename T, int OP>
+// RAGGED: rows of any length from 8,192 elements on and any 2-byte aligned base (an unpadded vocabulary): the vectors are
+// counted from the array's first 16-byte boundary, `head` elements in, so a tile starts at any column and the vector
+// that holds the end of one row and the start of the next takes the scalars of both; the fewer than 8 elements in
+// front of the first vector and behind the last one are transformed by the first lanes of workgroup 0 before its
+// first tile.  The array must hold fewer than 2^32 elements (the row of a tile comes from one 32-bit division).
+template <typename T, int OP, bool RAGGED>
 __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
     int32_t n, int64_t total_vec, int64_t ntiles, u32x4 *__restrict__ xv, const float *__restrict__ row_a,
     const float *__restrict__ row_b, const int32_t *__restrict__ target, uint32_t *__restrict__ tickets,
-    uint32_t *__restrict__ done_word, uint32_t launch_number) {
+    uint32_t *__restrict__ done_word, uint32_t launch_number, uint32_t head, uint32_t total) {
     constexpr int V = kFlatStreamVecs;
     constexpr int64_t kTileVecs = (int64_t)kFlatStreamThreads * V;
     struct Set {
@@ -688,11 +693,23 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
     const int64_t first = (int64_t)q * kFlatCounters + which;
     int64_t ahead = (int64_t)(q + (gridDim.x >> 3)) * kFlatCounters + which;
     const uint32_t drawn_base = 2u * (gridDim.x >> 3);      // the first two tiles of a workgroup follow from its number
+    if (RAGGED && blockIdx.x == 0) {     // the elements outside the vectors; no vector of any tile holds them
+        const uint32_t tail_lo = head + 8u * (uint32_t)total_vec;
+        const uint32_t nedge = head + (total - tail_lo);
+        if (threadIdx.x < nedge) {
+            uint16_t *x = (uint16_t *)xv - head;
+            const uint32_t i = threadIdx.x < head ? threadIdx.x : tail_lo + (threadIdx.x - head);
+            const uint32_t row = i / (uint32_t)n;
+            const int32_t col = (int32_t)(i - row * (uint32_t)n);
+            const bool is_t = OP == 0 ? (target[row] == col) : false;
+            x[i] = T::from_f32(flat_elem<T, OP>(T::to_f32(x[i]), is_t, row_a[row], flat_row_b<OP>(row_b, row)));
+        }
+    }
     if (first >= ntiles) { stream_slot_leave(tickets, done_word, launch_number); return; }
     uint32_t drawn = 0;
     if (threadIdx.x == 0) stream_draw(drawn, counter);
     const uint32_t row_vecs = (uint32_t)n >> 3;
-    const uint32_t last_row = (uint32_t)total_vec / row_vecs - 1;
+    const uint32_t last_row = RAGGED ? total / (uint32_t)n - 1 : (uint32_t)total_vec / row_vecs - 1;
 
     auto issue = [&](Set &s, int64_t tile_in) {
         s.real = tile_in < ntiles;
@@ -700,8 +717,15 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
         // loads of the per-row scalars below on the scalar unit, outside the vector memory counter
         const int64_t tile = s.real ? (int64_t)__builtin_amdgcn_readfirstlane((uint32_t)tile_in) : 0;
         s.base = tile * kTileVecs;
-        const uint32_t row0 = (uint32_t)s.base / row_vecs;       // the launcher keeps total_vec below 2^32
-        s.col0 = 8u * ((uint32_t)s.base - row0 * row_vecs);
+        uint32_t row0;
+        if (RAGGED) {
+            const uint32_t first_elem = head + 8u * (uint32_t)s.base;      // the launcher keeps the array below 2^32 elements
+            row0 = first_elem / (uint32_t)n;
+            s.col0 = first_elem - row0 * (uint32_t)n;
+        } else {
+            row0 = (uint32_t)s.base / row_vecs;                  // the launcher keeps total_vec below 2^32
+            s.col0 = 8u * ((uint32_t)s.base - row0 * row_vecs);
+        }
         const uint32_t row1 = row0 == last_row ? row0 : row0 + 1;     // the last row has no successor
         s.a0 = row_a[row0]; s.a1 = row_a[row1];
         if (OP == 0) { s.t0 = target[row0]; s.t1 = target[row1]; s.b0 = s.b1 = 0.f; }
@@ -719,16 +743,32 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
             const int64_t g = s.base + u * kFlatStreamThreads + threadIdx.x;
             if (g >= total_vec) continue;
             const uint32_t off = s.col0 + 8u * (uint32_t)(u * kFlatStreamThreads + threadIdx.x);
-            const bool next_row = off >= (uint32_t)n;
-            const int32_t col = (int32_t)(next_row ? off - (uint32_t)n : off);
-            const float a = next_row ? s.a1 : s.a0, b = next_row ? s.b1 : s.b0;
-            const int32_t tk = OP == 0 ? (next_row ? s.t1 : s.t0) - col : -1;
             u32x4 o;
+            if (RAGGED) {
+                // element k of the vector lies in the tile's first row while k < split, in the row after it otherwise
+                const int32_t split = n - (int32_t)off;
+                const int32_t tk0 = OP == 0 ? s.t0 - (int32_t)off : -1;       // position of either row's target in the vector
+                const int32_t tk1 = OP == 0 ? s.t1 + split : -1;
 #pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const float lo = flat_elem<T, OP>(lo_f32<T>(s.w[u][k]), tk == 2 * k, a, b);
-                const float hi = flat_elem<T, OP>(hi_f32<T>(s.w[u][k]), tk == 2 * k + 1, a, b);
-                o[k] = pack2<T>(lo, hi);
+                for (int k = 0; k < 4; k++) {
+                    const bool lo_next = 2 * k >= split, hi_next = 2 * k + 1 >= split;
+                    const float lo = flat_elem<T, OP>(lo_f32<T>(s.w[u][k]), (lo_next ? tk1 : tk0) == 2 * k,
+                                                      lo_next ? s.a1 : s.a0, lo_next ? s.b1 : s.b0);
+                    const float hi = flat_elem<T, OP>(hi_f32<T>(s.w[u][k]), (hi_next ? tk1 : tk0) == 2 * k + 1,
+                                                      hi_next ? s.a1 : s.a0, hi_next ? s.b1 : s.b0);
+                    o[k] = pack2<T>(lo, hi);
+                }
+            } else {
+                const bool next_row = off >= (uint32_t)n;
+                const int32_t col = (int32_t)(next_row ? off - (uint32_t)n : off);
+                const float a = next_row ? s.a1 : s.a0, b = next_row ? s.b1 : s.b0;
+                const int32_t tk = OP == 0 ? (next_row ? s.t1 : s.t0) - col : -1;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const float lo = flat_elem<T, OP>(lo_f32<T>(s.w[u][k]), tk == 2 * k, a, b);
+                    const float hi = flat_elem<T, OP>(hi_f32<T>(s.w[u][k]), tk == 2 * k + 1, a, b);
+                    o[k] = pack2<T>(lo, hi);
+                }
             }
             stream_store(xv + g, o);
         }
@@ -991,21 +1031,25 @@ static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void 
         int64_t tiles = (total_vec + kFlatThreads * kFlatUnroll - 1) / (kFlatThreads * kFlatUnroll);
         if (tiles < 1) tiles = 1;
         if (tiles > 0x7FFFFFFF) return fail(-1, "cross_entropy launcher: tensor too large for one launch");
-        if (n % 8 == 0 && head == 0 && n >= kFlatStreamMinRow && total_vec >= kFlatStreamMinVec && total_vec < ((int64_t)1 << 32)) {
+        const bool even = n % 8 == 0 && head == 0;
+        if (n >= kFlatStreamMinRow && total_vec >= kFlatStreamMinVec &&
+            (even ? total_vec < ((int64_t)1 << 32) : total < ((int64_t)1 << 32))) {
             StreamSlot fl;
             if (stream_slot_for(s, &fl, true)) {
                 uint32_t *tickets = fl.tickets;
                 const int cus = device_cu_count();
                 const unsigned grid = (unsigned)(cus >= 64 ? cus / 64 * 64 : 64);      // 8 XCDs x 8 counters
                 const int64_t per_tile = (int64_t)kFlatStreamThreads * kFlatStreamVecs;
-                hipLaunchKernelGGL((ce_flat_stream_kernel<T, OP>), dim3(grid), dim3(kFlatStreamThreads), 0, s, n, total_vec,
-                                   (total_vec + per_tile - 1) / per_tile, (u32x4 *)x, (const float *)row_a, (const float *)row_b,
-                                   (const int32_t *)target, tickets, fl.done_word, fl.number);
+                auto resident = even ? ce_flat_stream_kernel<T, OP, false> : ce_flat_stream_kernel<T, OP, true>;
+                hipLaunchKernelGGL(resident, dim3(grid), dim3(kFlatStreamThreads), 0, s, n, total_vec,
+                                   (total_vec + per_tile - 1) / per_tile, (u32x4 *)((uint16_t *)x + head), (const float *)row_a,
+                                   (const float *)row_b, (const int32_t *)target, tickets, fl.done_word, fl.number, (uint32_t)head,
+                                   (uint32_t)total);
                 hipError_t e = hipGetLastError();
                 return e == hipSuccess ? 0 : fail((int)e, who, e);
             }
         }
-        auto kern = (n % 8 == 0 && head == 0) ? ce_flat_vec_kernel<T, OP, false> : ce_flat_vec_kernel<T, OP, true>;
+        auto kern = even ? ce_flat_vec_kernel<T, OP, false> : ce_flat_vec_kernel<T, OP, true>;
         hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(kFlatThreads), 0, s, n, (int32_t)head, total_vec, total,
                            (uint16_t *)x, (const float *)row_a, (const float *)row_b, (const int32_t *)target);
     } else {

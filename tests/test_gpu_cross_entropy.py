@@ -226,13 +226,17 @@ def test_sumexp_and_softmax_inplace(name, dtype):
 
 
 @pytest.mark.parametrize("name,dtype", DTYPES)
-def test_elementwise_kernels_on_a_large_array(name, dtype):
+@pytest.mark.parametrize("m,n,off", [(4197, 32008, 0), (4200, 32001, 0), (4197, 32008, 3), (2700, 50257, 5), (1560, 86583, 0)])
+def test_elementwise_kernels_on_a_large_array(name, dtype, m, n, off):
     """Arrays of 2^27 elements or more with rows of 8,192 or more run as a resident grid whose tiles (8,192
-    elements) straddle rows and whose last tile is ragged: 4,197 rows of 32,008.  Backward is bit-exact on identical
-    input, the in-place softmax within one unit in the last place; two launches on two streams at once use separate
-    ticket counters; the words behind the array stay as they were."""
-    m, n = 4197, 32008
+    elements) straddle rows and whose last tile is ragged: 4,197 rows of 32,008; and, with vectors that hold the end
+    of one row and the start of the next and a few elements in front of the first vector and behind the last one, rows
+    whose length is not a multiple of 8 (32,001; 50,257; 86,583) and arrays that start `off` elements behind a 16-byte
+    boundary.  Backward is bit-exact on identical input, the in-place softmax within one unit in the last place; two
+    launches on two streams at once use separate ticket counters; the words in front of and behind the array stay
+    as they were."""
     assert m * n >= 1 << 27 and (m * n // 8) % 1024 != 0 and n % 8192 != 0
+    from bmtrain_amd import C
     x, t = _case(m, n, dtype, seed=77)
     soft, _ = oracle.ce_forward(bits16(x), t.numpy(), -100, name)
     v = (torch.rand(m, generator=torch.Generator().manual_seed(5)) * 32768.0 / m).float()
@@ -243,21 +247,23 @@ def test_elementwise_kernels_on_a_large_array(name, dtype):
     side = torch.cuda.Stream()
     bufs = []
     for _ in range(2):
-        buf = torch.full((m * n + guard,), 1.0, dtype=dtype, device="cuda")
-        buf[:m * n].view(m, n).copy_(from_bits16(soft, dtype).reshape(m, n))
+        buf = torch.full((off + m * n + guard,), 1.0, dtype=dtype, device="cuda")
+        buf[off:off + m * n].view(m, n).copy_(from_bits16(soft, dtype).reshape(m, n))
         bufs.append(buf)
     vg, tg = v.cuda(), t.cuda()
     torch.cuda.synchronize()
-    F.cross_entropy_backward_inplace(m, n, vg, tg, bufs[0][:m * n].view(m, n), -100)
+    before = C.bmt_hip_flat_stream_stats()
+    F.cross_entropy_backward_inplace(m, n, vg, tg, bufs[0][off:off + m * n].view(m, n), -100)
     with torch.cuda.stream(side):
-        F.cross_entropy_backward_inplace(m, n, vg, tg, bufs[1][:m * n].view(m, n), -100)
+        F.cross_entropy_backward_inplace(m, n, vg, tg, bufs[1][off:off + m * n].view(m, n), -100)
     torch.cuda.synchronize()
+    assert C.bmt_hip_flat_stream_stats()["resident"] == before["resident"] + 2      # both ran as the resident grid
     for buf in bufs:
-        assert np.array_equal(bits16(buf[:m * n]).reshape(m, n), want)
-        assert bool((buf[m * n:] == 1.0).all())
+        assert np.array_equal(bits16(buf[off:off + m * n]).reshape(m, n), want)
+        assert bool((buf[off + m * n:] == 1.0).all()) and bool((buf[:off] == 1.0).all())
 
     buf = bufs[0]
-    xg = buf[:m * n].view(m, n)
+    xg = buf[off:off + m * n].view(m, n)
     xg.copy_(x)
     mx = xg.float().max(-1).values.contiguous()
     want_se = oracle.fused_sumexp(bits16(x), mx.cpu().numpy(), name)
@@ -265,7 +271,7 @@ def test_elementwise_kernels_on_a_large_array(name, dtype):
     oracle.fused_softmax_inplace(want, mx.cpu().numpy(), want_se, name)
     F.fused_softmax_inplace(xg, mx, torch.from_numpy(want_se).cuda())
     assert ulp_distance16(bits16(xg), want).max() <= 1
-    assert bool((buf[m * n:] == 1.0).all())
+    assert bool((buf[off + m * n:] == 1.0).all()) and bool((buf[:off] == 1.0).all())
 
 
 def test_elementwise_kernels_on_more_streams_than_the_library_keeps_counters_for():

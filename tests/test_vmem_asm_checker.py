@@ -92,7 +92,7 @@ def test_the_bad_fixtures_differ_from_the_good_one_only_in_the_mistake():
 
 
 SHIPPED = (("adam.device.s", ["adam_stream_kernel", "adam_stream_multi_kernel"], 6),    # 2 flavours x 2 counter homes + 2 multi
-           ("cross_entropy.device.s", ["ce_flat_stream_kernel"], 4))
+           ("cross_entropy.device.s", ["ce_flat_stream_kernel"], 8))    # 2 types x 2 operations x rows on / off the vector grid
 
 
 @pytest.mark.parametrize("filename,wanted,expect", SHIPPED)
