@@ -127,12 +127,13 @@ __device__ __forceinline__ int64_t xcd_contiguous_row(uint32_t b, uint32_t rows)
     return b < whole ? (int64_t)(b & 7u) * (whole >> 3) + (b >> 3) : (int64_t)b;
 }
 
-// The same idea in runs: XCD k works through 32 consecutive rows, then through the 32 rows that lie 256 further on.
-// This is the order of the long-row kernel.  Measured against row = b on arrays of 2^29 elements, rows of 36,864 to
-// 151,936 classes: 0.4 to 9 % faster at fourteen of fifteen lengths (65,536: 3.3 %, 98,304: 6.4 %, 151,936: 2.9 %),
-// 0.3 % slower at 128,256; one run per XCD for the whole launch, as above, is ahead at some of these lengths and up to
-// 4 % behind at others, and runs of 8 or 128 rows gain less than runs of 32.
-constexpr uint32_t kXcdRunRows = 32;
+// The same idea in runs: XCD k works through 128 consecutive rows, then through the 128 rows that lie 1,024 further
+// on.  This is the order of the long-row kernel.  Measured against row = b, alternating in one process, on arrays of
+// 2^29 elements with rows of 36,864 to 151,936 classes: runs of 32, 64 and 128 rows are 2 % faster on average (65,536
+// classes: 2.8 %, 98,304: 5 to 6 %, 151,936: 2 to 3 %; never more than 1 % slower); at 8,192 x 128,256 runs of 128 are
+// 0.7 % faster (0.7453 against 0.7505 ms; runs of 32: 0.7515, of 64: 0.7484), runs of 8 are 1.3 % slower.  One run per
+// XCD for the whole launch, as above, is ahead at some lengths and up to 4 % behind at others.
+constexpr uint32_t kXcdRunRows = 128;
 __device__ __forceinline__ int64_t xcd_run_row(uint32_t b, uint32_t rows) {
     const uint32_t whole = rows / (8u * kXcdRunRows) * (8u * kXcdRunRows);
     if (b >= whole) return (int64_t)b;
