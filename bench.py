@@ -687,6 +687,8 @@ def main():
             "algorithmic_bytes_per_launch": ADAM_BF16_BYTES * n,
             "ms_per_launch": round(ms["adam"], 4),
             **spread("adam"),
+            # every timed launch in step order (the mean above is what `value` uses)
+            "ms_each_step": [round(ev[1].elapsed_time(ev[2]), 3) for ev in all_events],
         },
         "ce_fwd_bwd_rows_per_s": round(ce_rows_per_s, 1),
         "other_kernels": {
