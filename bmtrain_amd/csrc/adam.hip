@@ -276,6 +276,20 @@ __device__ __forceinline__ void stream_first_tickets(int &which, uint32_t &t0, u
     t0 = q;
     t1 = q + (gridDim.x >> 2);
 }
+// A workgroup takes its tiles from the counters in turn (its own, the next one, ...), so that all counters are drawn
+// from at the same rate whatever the pace of the single workgroups is.  With every workgroup on one counter of its
+// own the four interleaved tile sequences drift apart over a long launch when some compute units run slower than
+// others, the chip's window on the arrays widens, and launches over 6.74 B elements of a freshly allocated state took
+// 27.65 to 28.7 ms (mean 28.05); in turn: 27.34 to 27.37 ms, every launch (86.2 % of the HBM peak against 84 %; 2.4 to
+// 4.8 B elements: 87.5 against 85 %).  A counter's sequence only goes up, so a workgroup is done when it has met a tile
+// past the end from every counter in a row.
+// TURNS = false keeps every workgroup on its own counter (and lets it leave at its first tile past the end): launches
+// below 2^31 elements, which are over before the sequences have drifted, run up to 2 % faster that way, and short ones
+// save the three last draws (12.6 M elements: 3 to 5 %).
+template <bool TURNS>
+__device__ __forceinline__ int stream_next_counter(int c) { return TURNS ? (c + 1) & (kStreamCounters - 1) : c; }
+constexpr int64_t kStreamTurnsMinVec = (int64_t)1 << 29;       // 2^31 elements
+
 template <typename T>
 __global__ void adam_stream_finish_kernel(const f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, int64_t nvec) {
     if (threadIdx.x < kStreamCounters) {
@@ -299,7 +313,7 @@ struct StreamSet {
 // SLOT: the counters are a slot of the library's own array (stream_slot_for) instead of places in the 16-bit output;
 // every group then stores its 16-bit result, nothing runs in front of or behind the kernel, and the last workgroup to
 // leave puts the slot back (stream_slot_leave).
-template <bool FP16, bool SLOT>
+template <bool FP16, bool SLOT, bool TURNS>
 __global__ __launch_bounds__(kStreamThreads) void adam_stream_kernel(
     int64_t nvec, int64_t ntiles, f32x4 *__restrict__ p32, u32x2 *__restrict__ p16, const u32x2 *__restrict__ g16,
     typename MomentVec<FP16>::type *__restrict__ mom, f32x4 *__restrict__ var, AdamHyper h, uint32_t *__restrict__ slot,
@@ -310,15 +324,19 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_kernel(
     int which;
     uint32_t t0, t1;
     stream_first_tickets(which, t0, t1);
-    uint32_t *counter = SLOT ? slot + which * 1024 : (uint32_t *)(p16 + (nvec - 1 - which * kStreamCounterStride));
-    const uint32_t drawn_base = gridDim.x >> 1;                       // two tickets per workgroup are taken already
+    auto counter_of = [&](int c) -> uint32_t * {
+        return SLOT ? slot + c * 1024 : (uint32_t *)(p16 + (nvec - 1 - c * kStreamCounterStride));
+    };
+    const uint32_t drawn_base = gridDim.x >> 1;                       // two tickets per counter and workgroup of its group are taken already
     const int64_t first = (int64_t)t0 * kStreamCounters + which;
-    int64_t ahead = (int64_t)t1 * kStreamCounters + which;            // the tile after the one in flight
+    int64_t ahead = (int64_t)t1 * kStreamCounters + stream_next_counter<TURNS>(which);   // the tile after the one in flight
     if (first >= ntiles) {
         if (SLOT) stream_slot_leave(slot, done_word, launch_number);
         return;
     }
-    uint32_t drawn = 0;                                               // lane 0: ticket on its way
+    int drawing = stream_next_counter<TURNS>(stream_next_counter<TURNS>(which));    // counter of the ticket on its way
+    uint32_t *const counter = counter_of(drawing);                    // TURNS = false: the only one
+    uint32_t drawn = 0;                                               // lane 0: that ticket
     if (threadIdx.x == 0) stream_draw(drawn, counter);
 
     auto issue = [&](Set &s, int64_t tile) {
@@ -355,16 +373,32 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_kernel(
         asm volatile("s_waitcnt vmcnt(4)" : "+v"(cur.g), "+v"(cur.p), "+v"(cur.m), "+v"(cur.v), "+v"(drawn));
         if (threadIdx.x == 0) handed[turn] = drawn;
         __syncthreads();
-        ahead = (int64_t)(handed[turn] + drawn_base) * kStreamCounters + which;
-        if (threadIdx.x == 0) stream_draw(drawn, counter);
+        if constexpr (TURNS) {
+            ahead = (int64_t)(handed[turn] + drawn_base) * kStreamCounters + drawing;
+            drawing = stream_next_counter<TURNS>(drawing);
+            if (threadIdx.x == 0) stream_draw(drawn, counter_of(drawing));
+        } else {
+            ahead = (int64_t)(handed[turn] + drawn_base) * kStreamCounters + which;
+            if (threadIdx.x == 0) stream_draw(drawn, counter);
+        }
         finish(cur);
         return tile;
     };
     Set a, b;
     issue(a, first);
-    while (true) {
-        if (stage(a, b, 0) >= ntiles) break;
-        if (stage(b, a, 1) >= ntiles) break;
+    if constexpr (TURNS) {
+        int beyond = 0;  // tiles past the end in a row: one from every counter means that all counters have run out
+        while (true) {
+            beyond = stage(a, b, 0) >= ntiles ? beyond + 1 : 0;
+            if (beyond == kStreamCounters) break;
+            beyond = stage(b, a, 1) >= ntiles ? beyond + 1 : 0;
+            if (beyond == kStreamCounters) break;
+        }
+    } else {
+        while (true) {
+            if (stage(a, b, 0) >= ntiles) break;
+            if (stage(b, a, 1) >= ntiles) break;
+        }
     }
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");   // loads of the tile nobody owns, the last ticket
     if (SLOT) stream_slot_leave(slot, done_word, launch_number);
@@ -490,13 +524,15 @@ static hipError_t launch_bf16(int64_t n, float *p32, uint16_t *p16, const uint16
                 const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
                 StreamSlot slot;
                 if (stream_slot_for(s, &slot, false)) {
-                    hipLaunchKernelGGL((adam_stream_kernel<false, true>), dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
+                    auto kern = nvec >= kStreamTurnsMinVec ? adam_stream_kernel<false, true, true> : adam_stream_kernel<false, true, false>;
+                    hipLaunchKernelGGL(kern, dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
                                        ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (f32x4 *)(m + head),
                                        (f32x4 *)(v + head), h, slot.tickets, slot.done_word, slot.number);
                     return false;
                 }
                 hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec);
-                hipLaunchKernelGGL((adam_stream_kernel<false, false>), dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
+                auto hosted = nvec >= kStreamTurnsMinVec ? adam_stream_kernel<false, false, true> : adam_stream_kernel<false, false, false>;
+                hipLaunchKernelGGL(hosted, dim3(stream_grid()), dim3(kStreamThreads), 0, s, nvec,
                                    ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (f32x4 *)(m + head),
                                    (f32x4 *)(v + head), h, (uint32_t *)nullptr, (uint32_t *)nullptr, 0u);
                 hipLaunchKernelGGL((adam_stream_finish_kernel<BFloat16>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
@@ -529,13 +565,15 @@ static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16
                 const int64_t ntiles = (nvec + kStreamThreads - 1) / kStreamThreads;
                 StreamSlot slot;
                 if (stream_slot_for(s, &slot, false)) {
-                    hipLaunchKernelGGL((adam_stream_kernel<true, true>), dim3(stream_grid(true)), dim3(kStreamThreads), 0, s, nvec,
+                    auto kern = nvec >= kStreamTurnsMinVec ? adam_stream_kernel<true, true, true> : adam_stream_kernel<true, true, false>;
+                    hipLaunchKernelGGL(kern, dim3(stream_grid(true)), dim3(kStreamThreads), 0, s, nvec,
                                        ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
                                        (f32x4 *)(v + head), h, slot.tickets, slot.done_word, slot.number);
                     return false;
                 }
                 hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec);
-                hipLaunchKernelGGL((adam_stream_kernel<true, false>), dim3(stream_grid(true)), dim3(kStreamThreads), 0, s, nvec,
+                auto hosted = nvec >= kStreamTurnsMinVec ? adam_stream_kernel<true, false, true> : adam_stream_kernel<true, false, false>;
+                hipLaunchKernelGGL(hosted, dim3(stream_grid(true)), dim3(kStreamThreads), 0, s, nvec,
                                    ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
                                    (f32x4 *)(v + head), h, (uint32_t *)nullptr, (uint32_t *)nullptr, 0u);
                 hipLaunchKernelGGL((adam_stream_finish_kernel<Half>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
@@ -632,7 +670,7 @@ __global__ __launch_bounds__(kAdamThreads) void adam_multi_kernel(AdamBatch batc
 // argument (the tile is uniform, so the look-up runs on the scalar unit).  The four counters live in the
 // 16-bit output of batch.counter_tensor.  The elements that do not fill a 4-element group (up to three per
 // tensor) and the four vectors that hosted the counters are finished by adam_stream_multi_finish_kernel.
-template <bool FP16>
+template <bool FP16, bool TURNS>
 __global__ __launch_bounds__(kStreamThreads) void adam_stream_multi_kernel(AdamBatch batch, AdamHyper h) {
     typedef typename MomentVec<FP16>::type mom_t;
     typedef StreamSet<FP16> Set;
@@ -644,16 +682,21 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_multi_kernel(AdamB
     const int64_t ntiles = batch.stream_first[batch.count];
     const int ct = batch.counter_tensor;
     const int64_t ct_nvec = batch.n[ct] / 4;
-    uint32_t *counter = (uint32_t *)((u32x2 *)batch.p16[ct] + (ct_nvec - 1 - which * kStreamCounterStride));
+    auto counter_of = [&](int c) -> uint32_t * {
+        return (uint32_t *)((u32x2 *)batch.p16[ct] + (ct_nvec - 1 - c * kStreamCounterStride));
+    };
     const int64_t first = (int64_t)t0 * kStreamCounters + which;
-    int64_t ahead = (int64_t)t1 * kStreamCounters + which;
+    int64_t ahead = (int64_t)t1 * kStreamCounters + stream_next_counter<TURNS>(which);
     if (first >= ntiles) return;
+    int drawing = stream_next_counter<TURNS>(stream_next_counter<TURNS>(which));    // counter of the ticket on its way
+    uint32_t *const counter = counter_of(drawing);                    // TURNS = false: the only one
     uint32_t drawn = 0;
     if (threadIdx.x == 0) stream_draw(drawn, counter);
 
-    // The tiles a workgroup draws only ever go up, so the tensor of a tile is found by walking on from the
-    // tensor of the tile before, and its pointers are read from the kernel argument only when it changes;
-    // each register set remembers the pointers its tile was loaded through.
+    // The tiles of a workgroup stay close to each other (the counters move together, and each of them only goes up),
+    // so the tensor of a tile is found by walking from the tensor of the tile before, mostly not at all, and its
+    // pointers are read from the kernel argument only when it changes; each register set remembers the pointers its
+    // tile was loaded through.
     struct Where { float *p32; uint16_t *p16; const uint16_t *g16; void *mom; float *var; int64_t nvec; bool hosts_counters; };
     int t = 0;
     uint32_t t_first = 0, t_end = batch.stream_first[1];       // tensor t owns the tiles [t_first, t_end)
@@ -667,6 +710,7 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_multi_kernel(AdamB
             const uint32_t tile = __builtin_amdgcn_readfirstlane((uint32_t)tile_in);
             bool moved = false;
             while (tile >= t_end) { t++; t_first = t_end; t_end = batch.stream_first[t + 1]; moved = true; }
+            while (tile < t_first) { t--; t_end = t_first; t_first = batch.stream_first[t]; moved = true; }
             if (moved) cur_where = where_of(t);
             s.i = (int64_t)(tile - t_first) * kStreamThreads + threadIdx.x;
         } else {
@@ -703,16 +747,32 @@ __global__ __launch_bounds__(kStreamThreads) void adam_stream_multi_kernel(AdamB
         asm volatile("s_waitcnt vmcnt(4)" : "+v"(cur.g), "+v"(cur.p), "+v"(cur.m), "+v"(cur.v), "+v"(drawn));
         if (threadIdx.x == 0) handed[slot] = drawn;
         __syncthreads();
-        ahead = (int64_t)(handed[slot] + (gridDim.x >> 1)) * kStreamCounters + which;
-        if (threadIdx.x == 0) stream_draw(drawn, counter);
+        if constexpr (TURNS) {
+            ahead = (int64_t)(handed[slot] + (gridDim.x >> 1)) * kStreamCounters + drawing;
+            drawing = stream_next_counter<TURNS>(drawing);
+            if (threadIdx.x == 0) stream_draw(drawn, counter_of(drawing));
+        } else {
+            ahead = (int64_t)(handed[slot] + (gridDim.x >> 1)) * kStreamCounters + which;
+            if (threadIdx.x == 0) stream_draw(drawn, counter);
+        }
         finish(cur, wcur);
         return tile;
     };
     Set a, b;
     issue(a, wa, first);
-    while (true) {
-        if (stage(a, wa, b, wb, 0) >= ntiles) break;
-        if (stage(b, wb, a, wa, 1) >= ntiles) break;
+    if constexpr (TURNS) {
+        int beyond = 0;  // see adam_stream_kernel
+        while (true) {
+            beyond = stage(a, wa, b, wb, 0) >= ntiles ? beyond + 1 : 0;
+            if (beyond == kStreamCounters) break;
+            beyond = stage(b, wb, a, wa, 1) >= ntiles ? beyond + 1 : 0;
+            if (beyond == kStreamCounters) break;
+        }
+    } else {
+        while (true) {
+            if (stage(a, wa, b, wb, 0) >= ntiles) break;
+            if (stage(b, wb, a, wa, 1) >= ntiles) break;
+        }
     }
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
 }
@@ -802,8 +862,8 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
         }
         if (counters_clear && groups >= (FP16 ? kStreamMultiMinVecFp16 : kStreamMultiMinVecBf16)) {
             hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, (u32x2 *)batch.p16[batch.counter_tensor], most);
-            hipLaunchKernelGGL((adam_stream_multi_kernel<FP16>), dim3(stream_grid(FP16)), dim3(kStreamThreads), 0, s,
-                               batch, h);
+            auto resident = groups >= kStreamTurnsMinVec ? adam_stream_multi_kernel<FP16, true> : adam_stream_multi_kernel<FP16, false>;
+            hipLaunchKernelGGL(resident, dim3(stream_grid(FP16)), dim3(kStreamThreads), 0, s, batch, h);
             hipLaunchKernelGGL((adam_stream_multi_finish_kernel<FP16>), dim3(1), dim3(4 * kBatch + 64), 0, s, batch, h);
         } else {
             hipLaunchKernelGGL((adam_multi_kernel<FP16>), dim3(tiles), dim3(kAdamThreads), 0, s, batch, h);

@@ -685,7 +685,13 @@ static __device__ __align__(256) uint32_t flat_tickets[kFlatCounters * 1024];
 // that holds the end of one row and the start of the next takes the scalars of both; the fewer than 8 elements in
 // front of the first vector and behind the last one are transformed by the first lanes of workgroup 0 before its
 // first tile.  The array must hold fewer than 2^32 elements (the row of a tile comes from one 32-bit division).
-template <typename T, int OP, bool RAGGED>
+// TURNS: a workgroup takes its tiles from the counters in turn, as the long Adam launches do (see stream_next_counter in
+// adam.hip), so that all counters move at the same rate; it then leaves after it has met a tile past the end from
+// every counter in a row, seven draws later than with a counter of its own.  Measured against each other, alternating
+// in one process: 2^27 elements 78.2 against 81.0 % of peak, 2^28 82.0 / 82.8, 2^29 83.7 / 83.4, 16,384 x 32,000 83.7 / 83.2,
+// 8,192 x 128,256 84.5 / 83.7 - hence from 2^29 elements on.
+constexpr int64_t kFlatTurnsMinVec = (int64_t)1 << 26;
+template <typename T, int OP, bool RAGGED, bool TURNS>
 __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
     int32_t n, int64_t total_vec, int64_t ntiles, u32x4 *__restrict__ xv, const float *__restrict__ row_a,
     const float *__restrict__ row_b, const int32_t *__restrict__ target, uint32_t *__restrict__ tickets,
@@ -703,9 +709,9 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
     __shared__ uint32_t handed[2];
     const int which = (int)((blockIdx.x >> 3) & (kFlatCounters - 1));
     const uint32_t q = ((blockIdx.x >> 6) << 3) | (blockIdx.x & 7u);      // number among the workgroups of this counter
-    uint32_t *counter = tickets + which * 1024;
+    auto next_counter = [](int c) { return TURNS ? (c + 1) & (kFlatCounters - 1) : c; };
     const int64_t first = (int64_t)q * kFlatCounters + which;
-    int64_t ahead = (int64_t)(q + (gridDim.x >> 3)) * kFlatCounters + which;
+    int64_t ahead = (int64_t)(q + (gridDim.x >> 3)) * kFlatCounters + next_counter(which);
     const uint32_t drawn_base = 2u * (gridDim.x >> 3);      // the first two tiles of a workgroup follow from its number
     if (RAGGED && blockIdx.x == 0) {     // the elements outside the vectors; no vector of any tile holds them
         const uint32_t tail_lo = head + 8u * (uint32_t)total_vec;
@@ -720,6 +726,8 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
         }
     }
     if (first >= ntiles) { stream_slot_leave(tickets, done_word, launch_number); return; }
+    int drawing = next_counter(next_counter(which));        // counter of the ticket on its way
+    uint32_t *const counter = tickets + drawing * 1024;     // TURNS = false: the only one
     uint32_t drawn = 0;
     if (threadIdx.x == 0) stream_draw(drawn, counter);
     const uint32_t row_vecs = (uint32_t)n >> 3;
@@ -793,16 +801,32 @@ __global__ __launch_bounds__(kFlatStreamThreads) void ce_flat_stream_kernel(
         asm volatile("s_waitcnt vmcnt(4)" : "+v"(cur.w[0]), "+v"(cur.w[1]), "+v"(cur.w[2]), "+v"(cur.w[3]), "+v"(drawn));
         if (threadIdx.x == 0) handed[slot] = drawn;
         __syncthreads();
-        ahead = (int64_t)(handed[slot] + drawn_base) * kFlatCounters + which;
-        if (threadIdx.x == 0) stream_draw(drawn, counter);
+        if constexpr (TURNS) {
+            ahead = (int64_t)(handed[slot] + drawn_base) * kFlatCounters + drawing;
+            drawing = next_counter(drawing);
+            if (threadIdx.x == 0) stream_draw(drawn, tickets + drawing * 1024);
+        } else {
+            ahead = (int64_t)(handed[slot] + drawn_base) * kFlatCounters + which;
+            if (threadIdx.x == 0) stream_draw(drawn, counter);
+        }
         finish(cur);
         return tile;
     };
     Set a, b;
     issue(a, first);
-    while (true) {
-        if (stage(a, b, 0) >= ntiles) break;
-        if (stage(b, a, 1) >= ntiles) break;
+    if constexpr (TURNS) {
+        int beyond = 0;  // tiles past the end in a row: one from every counter means that all counters have run out
+        while (true) {
+            beyond = stage(a, b, 0) >= ntiles ? beyond + 1 : 0;
+            if (beyond == kFlatCounters) break;
+            beyond = stage(b, a, 1) >= ntiles ? beyond + 1 : 0;
+            if (beyond == kFlatCounters) break;
+        }
+    } else {
+        while (true) {
+            if (stage(a, b, 0) >= ntiles) break;
+            if (stage(b, a, 1) >= ntiles) break;
+        }
     }
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
     stream_slot_leave(tickets, done_word, launch_number);
@@ -1054,7 +1078,9 @@ static int ce_flat(int32_t m, int32_t n, void *x, const void *row_a, const void 
                 const int cus = device_cu_count();
                 const unsigned grid = (unsigned)(cus >= 64 ? cus / 64 * 64 : 64);      // 8 XCDs x 8 counters
                 const int64_t per_tile = (int64_t)kFlatStreamThreads * kFlatStreamVecs;
-                auto resident = even ? ce_flat_stream_kernel<T, OP, false> : ce_flat_stream_kernel<T, OP, true>;
+                const bool turns = total_vec >= kFlatTurnsMinVec;
+                auto resident = even ? (turns ? ce_flat_stream_kernel<T, OP, false, true> : ce_flat_stream_kernel<T, OP, false, false>)
+                                     : (turns ? ce_flat_stream_kernel<T, OP, true, true> : ce_flat_stream_kernel<T, OP, true, false>);
                 hipLaunchKernelGGL(resident, dim3(grid), dim3(kFlatStreamThreads), 0, s, n, total_vec,
                                    (total_vec + per_tile - 1) / per_tile, (u32x4 *)((uint16_t *)x + head), (const float *)row_a,
                                    (const float *)row_b, (const int32_t *)target, tickets, fl.done_word, fl.number, (uint32_t)head,

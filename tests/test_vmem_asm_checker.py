@@ -91,8 +91,8 @@ def test_the_bad_fixtures_differ_from_the_good_one_only_in_the_mistake():
     assert body("vmem_ends_with_load_in_flight.s") == [l for l in good if l != "\ts_waitcnt vmcnt(0)"]
 
 
-SHIPPED = (("adam.device.s", ["adam_stream_kernel", "adam_stream_multi_kernel"], 6),    # 2 flavours x 2 counter homes + 2 multi
-           ("cross_entropy.device.s", ["ce_flat_stream_kernel"], 8))    # 2 types x 2 operations x rows on / off the vector grid
+SHIPPED = (("adam.device.s", ["adam_stream_kernel", "adam_stream_multi_kernel"], 12),   # (2 flavours x 2 counter homes + 2 multi) x counters fixed / in turn
+           ("cross_entropy.device.s", ["ce_flat_stream_kernel"], 16))   # 2 types x 2 operations x rows on / off the vector grid x counters fixed / in turn
 
 
 @pytest.mark.parametrize("filename,wanted,expect", SHIPPED)
