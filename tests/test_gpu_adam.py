@@ -453,6 +453,46 @@ def test_long_multi_tensor_launch_runs_as_one_resident_grid(flavour):
                                    y.view(torch.int16 if y.element_size() == 2 else torch.int32))
 
 
+@pytest.mark.parametrize("flavour", ["bf16", "fp16"])
+def test_multi_tensor_launch_of_more_than_2_to_the_31_elements(flavour):
+    """A batch of 2^31 elements or more takes its tiles from the four counters in turn, and a workgroup's tiles may then
+    step back over a tensor boundary.  Five tensors of 3 to 1.2 B elements (2.4 B in all, every leftover count, the
+    largest one - which hosts the counters - in the middle) in one multi-tensor launch against one launch per tensor,
+    by checksum of every array and bit for bit on a slice around every tensor's end."""
+    dt16 = torch.float16 if flavour == "fp16" else torch.bfloat16
+    mdt = torch.float16 if flavour == "fp16" else torch.float32
+    fn = F.adam_fp16 if flavour == "fp16" else F.adam_bf16
+    sizes = [900_000_001, 3, 1_200_000_002, 4099, 300_000_003]
+    assert sum(sizes) >= 1 << 31
+    gen = torch.Generator(device="cuda").manual_seed(9)
+
+    def filled(n, std, dtype, absolute=False):
+        x = torch.empty(n, dtype=dtype, device="cuda")
+        for lo in range(0, n, 1 << 27):
+            part = x[lo:lo + (1 << 27)]
+            r = torch.randn(part.numel(), generator=gen, device="cuda") * std
+            part.copy_(r.abs() if absolute else r)
+        return x
+    single, multi = [], []
+    for n in sizes:
+        p, m = filled(n, 0.02, torch.float32), filled(n, 1e-4, mdt)
+        v, g = filled(n, 1e-6, torch.float32, absolute=True), filled(n, 1e-3, dt16)
+        single.append((p, torch.full((n,), -1, dtype=dt16, device="cuda"), g, m, v))
+        multi.append((p.clone(), torch.full((n,), -1, dtype=dt16, device="cuda"), g, m.clone(), v.clone()))
+    for p32, p16, g, m, v in single:
+        fn(p32, p16, g, m, v, 0.9, 0.999, 1e-8, 1e-3, 2.0, 0.01, 5)
+    F.adam_multi(multi, 0.9, 0.999, 1e-8, 1e-3, 2.0, 0.01, 5)
+    torch.cuda.synchronize()
+    for a, b in zip(single, multi):
+        for k in (0, 1, 3, 4):
+            x, y = a[k], b[k]
+            assert _checksum(x) == _checksum(y), k
+            kind = torch.int16 if x.element_size() == 2 else torch.int32
+            assert torch.equal(x[-70_000:].view(kind), y[-70_000:].view(kind)) and torch.equal(x[:70_000].view(kind), y[:70_000].view(kind))
+    del single, multi
+    torch.cuda.empty_cache()
+
+
 def _checksum(t, chunk=1 << 28):
     """Order-independent 64-bit checksum of a tensor's bit patterns."""
     view = t.view(torch.int32 if t.element_size() == 4 else torch.int16)
