@@ -650,7 +650,7 @@ def main():
 
     def spread(name):
         ts = per_step[name]
-        return {"ms_median": round(ts[len(ts) // 2], 4), "ms_min": round(ts[0], 4)}
+        return {"ms_median": round(ts[len(ts) // 2], 4), "ms_min": round(ts[0], 4), "ms_max": round(ts[-1], 4)}
     adam_gbps = ADAM_BF16_BYTES * n / (ms["adam"] * 1e-3) / 1e9
     scan_gbps = SCAN_BYTES * n / (ms["has_inf_nan"] * 1e-3) / 1e9
     ce_ms = ms["ce_forward"] + ms["ce_backward"]

@@ -263,9 +263,12 @@ __global__ void adam_stream_reset_kernel(u32x2 *p16, int64_t nvec) {
 // The fp16 flavour moves fewer bytes per tile (its first moment is a 16-bit array) and runs 1 % faster with a
 // quarter more workgroups (1.6 B elements: 81.3 % of peak with 320 workgroups, 80.1 % with 256, 80.6 % with 384, 78 % with
 // 512); the bf16 flavour is fastest with exactly one per compute unit (84 %; 288: 82 %, 320: 81 %).
-static unsigned stream_grid(bool fp16 = false) {
+// With the counters taken in turn (launches of 2^31 elements or more) the fp16 flavour is fastest with two per compute
+// unit (6.74 B elements: 83.7 % with 512 workgroups, 83.2 % with 320 or 384, 82.1 % with 256; bf16: 84.6 % with 256,
+// 84.1 % with 288, 83.2 % with 512).
+static unsigned stream_grid(bool fp16 = false, bool turns = false) {
     int cus = device_cu_count();
-    if (fp16) cus += cus / 4;
+    if (fp16) cus += turns ? cus : cus / 4;
     return (unsigned)(cus >= 32 ? cus / 32 * 32 : 32);
 }
 // Workgroup b draws from counter (b / 8) % 4.  Its first two tickets need no atomic: it is workgroup number q
@@ -566,14 +569,14 @@ static hipError_t launch_fp16(int64_t n, float *p32, uint16_t *p16, const uint16
                 StreamSlot slot;
                 if (stream_slot_for(s, &slot, false)) {
                     auto kern = nvec >= kStreamTurnsMinVec ? adam_stream_kernel<true, true, true> : adam_stream_kernel<true, true, false>;
-                    hipLaunchKernelGGL(kern, dim3(stream_grid(true)), dim3(kStreamThreads), 0, s, nvec,
+                    hipLaunchKernelGGL(kern, dim3(stream_grid(true, nvec >= kStreamTurnsMinVec)), dim3(kStreamThreads), 0, s, nvec,
                                        ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
                                        (f32x4 *)(v + head), h, slot.tickets, slot.done_word, slot.number);
                     return false;
                 }
                 hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, out16, nvec);
                 auto hosted = nvec >= kStreamTurnsMinVec ? adam_stream_kernel<true, false, true> : adam_stream_kernel<true, false, false>;
-                hipLaunchKernelGGL(hosted, dim3(stream_grid(true)), dim3(kStreamThreads), 0, s, nvec,
+                hipLaunchKernelGGL(hosted, dim3(stream_grid(true, nvec >= kStreamTurnsMinVec)), dim3(kStreamThreads), 0, s, nvec,
                                    ntiles, (f32x4 *)(p32 + head), out16, (const u32x2 *)(g + head), (u32x2 *)(m + head),
                                    (f32x4 *)(v + head), h, (uint32_t *)nullptr, (uint32_t *)nullptr, 0u);
                 hipLaunchKernelGGL((adam_stream_finish_kernel<Half>), dim3(1), dim3(64), 0, s, (const f32x4 *)(p32 + head),
@@ -863,7 +866,7 @@ static int adam_multi(int32_t count, const bmt_adam_tensor *tensors, const AdamH
         if (counters_clear && groups >= (FP16 ? kStreamMultiMinVecFp16 : kStreamMultiMinVecBf16)) {
             hipLaunchKernelGGL(adam_stream_reset_kernel, dim3(1), dim3(64), 0, s, (u32x2 *)batch.p16[batch.counter_tensor], most);
             auto resident = groups >= kStreamTurnsMinVec ? adam_stream_multi_kernel<FP16, true> : adam_stream_multi_kernel<FP16, false>;
-            hipLaunchKernelGGL(resident, dim3(stream_grid(FP16)), dim3(kStreamThreads), 0, s, batch, h);
+            hipLaunchKernelGGL(resident, dim3(stream_grid(FP16, groups >= kStreamTurnsMinVec)), dim3(kStreamThreads), 0, s, batch, h);
             hipLaunchKernelGGL((adam_stream_multi_finish_kernel<FP16>), dim3(1), dim3(4 * kBatch + 64), 0, s, batch, h);
         } else {
             hipLaunchKernelGGL((adam_multi_kernel<FP16>), dim3(tiles), dim3(kAdamThreads), 0, s, batch, h);
