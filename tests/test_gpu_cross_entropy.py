@@ -226,7 +226,8 @@ def test_sumexp_and_softmax_inplace(name, dtype):
 
 
 @pytest.mark.parametrize("name,dtype", DTYPES)
-@pytest.mark.parametrize("m,n,off", [(4197, 32008, 0), (4200, 32001, 0), (4197, 32008, 3), (2700, 50257, 5), (1560, 86583, 0)])
+@pytest.mark.parametrize("m,n,off", [(4197, 32008, 0), (4200, 32001, 0), (4197, 32008, 3), (2700, 50257, 5), (1560, 86583, 0),
+                                     (16800, 32001, 5)])      # 2^29 elements or more: the counters are taken in turn
 def test_elementwise_kernels_on_a_large_array(name, dtype, m, n, off):
     """Arrays of 2^27 elements or more with rows of 8,192 or more run as a resident grid whose tiles (8,192
     elements) straddle rows and whose last tile is ragged: 4,197 rows of 32,008; and, with vectors that hold the end
